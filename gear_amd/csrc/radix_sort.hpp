@@ -1,0 +1,182 @@
+// Stable least-significant-digit radix sort (8-bit digits) for key/value pairs, gfx950.
+//
+// Per digit: (1) every tile counts its digits in an LDS histogram, (2) one workgroup turns the
+// digit-major table of tile counts into global offsets, (3) every tile re-reads its keys, ranks
+// them in LDS (wave ballots give the rank among equal digits inside a wave, a small LDS table
+// the rank across the waves of the tile) and scatters keys and payloads to their final place for
+// this digit.  Ranks follow element order, so the sort is stable.
+#pragma once
+#include "wave.hpp"
+
+namespace gearhip {
+namespace radix {
+namespace {  // every translation unit gets its own copy of the kernels
+
+constexpr int kBlock = 256;
+constexpr int kBins = 256;
+constexpr int kWaves = kBlock / kWave;
+constexpr int kScanBlock = 1024;
+
+struct Plan {
+  int rounds;      // elements per thread and tile
+  int64_t ntiles;  // tiles of kBlock * rounds elements
+};
+
+inline Plan plan(int64_t num) {
+  Plan p;
+  int64_t r = ceil_div64(num, (int64_t)kBlock * 1024);
+  if (r < 4) r = 4;
+  if (r > 64) r = 64;
+  p.rounds = (int)r;
+  p.ntiles = num <= 0 ? 0 : ceil_div64(num, (int64_t)kBlock * r);
+  return p;
+}
+
+inline size_t hist_bytes(int64_t num) {
+  return align_up((size_t)plan(num).ntiles * kBins * sizeof(uint32_t) + 256, 256);
+}
+
+template <typename K>
+__global__ __launch_bounds__(kBlock) void hist_kernel(const K *__restrict__ keys, int64_t num,
+                                                      int shift, int rounds, int64_t ntiles,
+                                                      uint32_t *__restrict__ hist) {
+  __shared__ uint32_t h[kBins];
+  const int tid = threadIdx.x;
+  h[tid] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kBlock * rounds;
+  for (int r = 0; r < rounds; ++r) {
+    const int64_t i = base + (int64_t)r * kBlock + tid;
+    if (i < num) atomicAdd(&h[(uint32_t)(keys[i] >> shift) & 255u], 1u);
+  }
+  __syncthreads();
+  hist[(int64_t)tid * ntiles + blockIdx.x] = h[tid];
+}
+
+// Exclusive scan of m counters in place, one workgroup.
+__global__ __launch_bounds__(kScanBlock) void hist_scan_kernel(uint32_t *h, int64_t m) {
+  __shared__ uint32_t wsum[kScanBlock / kWave];
+  __shared__ uint32_t carry;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int64_t base = 0; base < m; base += kScanBlock) {
+    const int64_t i = base + tid;
+    const int v = i < m ? (int)h[i] : 0;
+    const int inc = wave_inclusive_sum(v);
+    if (lane == 63) wsum[wave] = (uint32_t)inc;
+    __syncthreads();
+    uint32_t before = carry, total = 0;
+    for (int w = 0; w < kScanBlock / kWave; ++w) {
+      if (w < wave) before += wsum[w];
+      total += wsum[w];
+    }
+    if (i < m) h[i] = before + (uint32_t)(inc - v);
+    __syncthreads();
+    if (tid == 0) carry += total;
+    __syncthreads();
+  }
+}
+
+template <typename K, typename V, bool HAS_V>
+__global__ __launch_bounds__(kBlock) void scatter_kernel(const K *__restrict__ kin,
+                                                         const V *__restrict__ vin,
+                                                         K *__restrict__ kout,
+                                                         V *__restrict__ vout, int64_t num,
+                                                         int shift, int rounds, int64_t ntiles,
+                                                         const uint32_t *__restrict__ offsets) {
+  __shared__ uint32_t base[kBins];
+  __shared__ uint32_t wcnt[kWaves][kBins];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  base[tid] = offsets[(int64_t)tid * ntiles + blockIdx.x];
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) wcnt[w][tid] = 0;
+  __syncthreads();
+  const int64_t tile0 = (int64_t)blockIdx.x * kBlock * rounds;
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  for (int r = 0; r < rounds; ++r) {
+    const int64_t i = tile0 + (int64_t)r * kBlock + tid;
+    const bool valid = i < num;
+    const K key = valid ? kin[i] : (K)0;
+    const uint32_t d = (uint32_t)(key >> shift) & 255u;
+    uint64_t peers = wave_ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const bool bit = (d >> b) & 1u;
+      const uint64_t bal = wave_ballot(bit);
+      peers &= bit ? bal : ~bal;
+    }
+    const int rank = __popcll(peers & lt_mask);
+    if (valid && rank == 0) wcnt[wave][d] = (uint32_t)__popcll(peers);
+    __syncthreads();
+    if (valid) {
+      uint32_t pos = base[d] + (uint32_t)rank;
+      for (int w = 0; w < wave; ++w) pos += wcnt[w][d];
+      kout[pos] = key;
+      if (HAS_V) vout[pos] = vin[i];
+    }
+    __syncthreads();
+    {
+      uint32_t s = 0;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        s += wcnt[w][tid];
+        wcnt[w][tid] = 0;
+      }
+      base[tid] += s;
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T>
+__global__ void copy_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t num) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < num) out[i] = in[i];
+}
+
+// Sorts bits [begin_bit, end_bit) of the keys ascending, stable.  kin/vin are not modified; the
+// result lands in kout/vout; ktmp/vtmp are scratch of the same size; hist has hist_bytes(num).
+// vin == nullptr sorts keys only.  num < 2^32.
+template <typename K, typename V>
+int sort_pairs(const K *kin, K *kout, const V *vin, V *vout, K *ktmp, V *vtmp, int64_t num,
+               int begin_bit, int end_bit, uint32_t *hist, hipStream_t st) {
+  if (num <= 0) return 0;
+  if (num >= (1ll << 32)) return GEAR_HIP_ERANGE;
+  const Plan p = plan(num);
+  const int passes = end_bit > begin_bit ? (end_bit - begin_bit + 7) / 8 : 0;
+  const bool has_v = vin != nullptr;
+  if (passes == 0) {
+    const unsigned g = (unsigned)ceil_div64(num, 256);
+    copy_kernel<K><<<dim3(g), dim3(256), 0, st>>>(kin, kout, num);
+    if (has_v) copy_kernel<V><<<dim3(g), dim3(256), 0, st>>>(vin, vout, num);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  const K *ksrc = kin;
+  const V *vsrc = vin;
+  bool to_out = (passes & 1) != 0;  // alternate so that the last pass writes kout/vout
+  for (int pass = 0; pass < passes; ++pass) {
+    const int shift = begin_bit + 8 * pass;
+    K *kdst = to_out ? kout : ktmp;
+    V *vdst = to_out ? vout : vtmp;
+    hist_kernel<K><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(ksrc, num, shift, p.rounds,
+                                                                     p.ntiles, hist);
+    hist_scan_kernel<<<dim3(1), dim3(kScanBlock), 0, st>>>(hist, p.ntiles * kBins);
+    if (has_v)
+      scatter_kernel<K, V, true><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(
+          ksrc, vsrc, kdst, vdst, num, shift, p.rounds, p.ntiles, hist);
+    else
+      scatter_kernel<K, V, false><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(
+          ksrc, vsrc, kdst, vdst, num, shift, p.rounds, p.ntiles, hist);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    ksrc = kdst;
+    vsrc = vdst;
+    to_out = !to_out;
+  }
+  return 0;
+}
+
+}  // namespace
+}  // namespace radix
+}  // namespace gearhip

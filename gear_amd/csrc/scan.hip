@@ -1,0 +1,280 @@
+// Single-pass inclusive prefix sum (decoupled look-back) and a deterministic sum, gfx950.
+//
+// A tile is 256 threads x 4 rows of 16-byte input vectors, read with the lanes of a wave on
+// consecutive vectors (coalesced).  Each thread scans inside its vectors, the four row sums go
+// through a DPP wave scan, wave totals meet in LDS, and the tile's exclusive prefix comes from the
+// tiles before it through two 64-bit words per tile in the workspace:
+//     aggr[t]  sum of tile t alone            incl[t]  sum of tiles 0..t
+// A word equal to kEmpty means "not published yet"; value and readiness travel in one agent-scope
+// 64-bit store, so no fence pairs are needed.  Tile numbers are handed out by an atomic ticket in
+// launch order, hence every predecessor a tile waits for is already running.
+// Wave 0 of a tile looks back 64 predecessors at a time (one per lane, ballots pick the nearest
+// published inclusive value).  fp32 inputs are accumulated in fp64.
+#include "wave.hpp"
+
+namespace gearhip {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kRows = 4;
+constexpr uint64_t kEmpty = ~0ull;  // not a sum of fp32-derived doubles, not a non-negative int64
+constexpr size_t kHeaderBytes = 256;
+
+template <typename Acc> struct Bits;
+template <> struct Bits<double> {
+  static __device__ __forceinline__ uint64_t to(double v) { return (uint64_t)__double_as_longlong(v); }
+  static __device__ __forceinline__ double from(uint64_t b) { return __longlong_as_double((long long)b); }
+};
+template <> struct Bits<int64_t> {
+  static __device__ __forceinline__ uint64_t to(int64_t v) { return (uint64_t)v; }
+  static __device__ __forceinline__ int64_t from(uint64_t b) { return (int64_t)b; }
+};
+
+template <typename In, int VE> struct InVec;
+template <> struct InVec<float, 4> {
+  typedef float type __attribute__((ext_vector_type(4), aligned(4)));
+};
+template <> struct InVec<int64_t, 2> {
+  typedef int64_t type __attribute__((ext_vector_type(2), aligned(8)));
+};
+template <typename Acc> struct OutVec2;
+template <> struct OutVec2<double> {
+  typedef double type __attribute__((ext_vector_type(2), aligned(8)));
+};
+template <> struct OutVec2<int64_t> {
+  typedef int64_t type __attribute__((ext_vector_type(2), aligned(8)));
+};
+
+__global__ void scan_init_kernel(uint32_t *ticket, uint64_t *desc, int64_t words) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i == 0) *ticket = 0u;
+  if (i < words) desc[i] = kEmpty;
+}
+
+template <typename In, typename Acc, int VE>
+__global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
+                                                      Acc *__restrict__ out, int64_t n,
+                                                      uint32_t *ticket, uint64_t *aggr,
+                                                      uint64_t *incl) {
+  constexpr int kTileElems = kRows * kBlock * VE;
+  constexpr int kWaves = kBlock / kWave;
+  typedef typename InVec<In, VE>::type in_vec;
+  typedef typename OutVec2<Acc>::type out_vec2;
+  __shared__ Acc wtot[kRows][kWaves];
+  __shared__ Acc s_excl;
+  __shared__ uint32_t s_tile;
+
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+  __syncthreads();
+  const int64_t tile = s_tile;
+  const int64_t base = tile * kTileElems;
+
+  Acc x[kRows][VE];
+  Acc s[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
+    if (e0 + VE <= n) {
+      const in_vec v = *reinterpret_cast<const in_vec *>(in + e0);
+#pragma unroll
+      for (int j = 0; j < VE; ++j) x[r][j] = (Acc)v[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < VE; ++j) x[r][j] = (e0 + j < n) ? (Acc)in[e0 + j] : (Acc)0;
+    }
+#pragma unroll
+    for (int j = 1; j < VE; ++j) x[r][j] += x[r][j - 1];
+    s[r] = x[r][VE - 1];
+  }
+
+  Acc wexcl[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const Acc inc = wave_inclusive_sum(s[r]);
+    wexcl[r] = wave_shift_up1(inc);
+    if (lane == kWave - 1) wtot[r][wave] = inc;
+  }
+  __syncthreads();
+
+  Acc tile_total = (Acc)0;
+  Acc mybase[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    Acc acc = tile_total;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      if (w == wave) mybase[r] = acc + wexcl[r];
+      acc += wtot[r][w];
+    }
+    tile_total = acc;
+  }
+
+  if (wave == 0) {
+    Acc excl = (Acc)0;
+    if (tile == 0) {
+      if (lane == 0) store_agent(&incl[0], Bits<Acc>::to(tile_total));
+    } else {
+      if (lane == 0) store_agent(&aggr[tile], Bits<Acc>::to(tile_total));
+      int64_t look = tile - 1;
+      while (true) {
+        const int64_t idx = look - lane;
+        uint64_t vi = kEmpty, va = kEmpty;
+        if (idx >= 0) {
+          vi = load_agent(&incl[idx]);
+          if (vi == kEmpty) va = load_agent(&aggr[idx]);
+        }
+        const bool has_incl = (idx < 0) || (vi != kEmpty);
+        const bool ready = has_incl || (va != kEmpty);
+        const uint64_t bi = wave_ballot(has_incl), br = wave_ballot(ready);
+        const int first = bi ? (__ffsll((unsigned long long)bi) - 1) : kWave;
+        const uint64_t need = first >= 63 ? ~0ull : ((2ull << first) - 1ull);
+        if ((br & need) != need) {
+          __builtin_amdgcn_s_sleep(1);
+          continue;
+        }
+        Acc c = (Acc)0;
+        if (lane < first)
+          c = Bits<Acc>::from(va);
+        else if (lane == first && idx >= 0)
+          c = Bits<Acc>::from(vi);
+        excl += wave_sum(c);
+        if (first < kWave) break;
+        look -= kWave;
+      }
+      if (lane == 0) store_agent(&incl[tile], Bits<Acc>::to(excl + tile_total));
+    }
+    if (lane == 0) s_excl = excl;
+  }
+  __syncthreads();
+  const Acc excl = s_excl;
+
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
+    const Acc b = excl + mybase[r];
+    if (e0 + VE <= n) {
+#pragma unroll
+      for (int j = 0; j < VE; j += 2) {
+        out_vec2 o;
+        o[0] = b + x[r][j];
+        o[1] = b + x[r][j + 1];
+        *reinterpret_cast<out_vec2 *>(out + e0 + j) = o;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VE; ++j)
+        if (e0 + j < n) out[e0 + j] = b + x[r][j];
+    }
+  }
+}
+
+// ---- deterministic sum: fixed grid, fixed tree ------------------------------------------------
+constexpr int kSumMaxBlocks = 1024;
+
+__global__ __launch_bounds__(kBlock) void sum_partial_kernel(const float *__restrict__ in,
+                                                             int64_t n, double *partial) {
+  __shared__ double wtot[kBlock / kWave];
+  typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
+  const int tid = threadIdx.x;
+  double acc = 0.0;
+  const int64_t nvec = n >> 2;
+  for (int64_t v = (int64_t)blockIdx.x * kBlock + tid; v < nvec; v += (int64_t)gridDim.x * kBlock) {
+    const f4 q = *reinterpret_cast<const f4 *>(in + (v << 2));
+    acc += ((double)q[0] + (double)q[1]) + ((double)q[2] + (double)q[3]);
+  }
+  if (blockIdx.x == 0 && tid < (int)(n & 3)) acc += (double)in[(nvec << 2) + tid];
+  const double w = wave_sum(acc);
+  if ((tid & 63) == 0) wtot[tid >> 6] = w;
+  __syncthreads();
+  if (tid == 0) partial[blockIdx.x] = (wtot[0] + wtot[1]) + (wtot[2] + wtot[3]);
+}
+
+__global__ __launch_bounds__(kBlock) void sum_final_kernel(const double *partial, int nblocks,
+                                                           float *out, double *out_f64) {
+  __shared__ double wtot[kBlock / kWave];
+  const int tid = threadIdx.x;
+  double acc = 0.0;
+  for (int i = tid; i < nblocks; i += kBlock) acc += partial[i];
+  const double w = wave_sum(acc);
+  if ((tid & 63) == 0) wtot[tid >> 6] = w;
+  __syncthreads();
+  if (tid == 0) {
+    const double t = (wtot[0] + wtot[1]) + (wtot[2] + wtot[3]);
+    if (out) *out = (float)t;
+    if (out_f64) *out_f64 = t;
+  }
+}
+
+int64_t scan_tiles(int64_t n, int tile_elems) { return n <= 0 ? 0 : ceil_div64(n, tile_elems); }
+
+// the workspace is sized for the smaller tile (int64: 2048 elements) so both scans fit
+size_t scan_ws_bytes(int64_t n) {
+  const int64_t tiles = scan_tiles(n, kRows * kBlock * 2);
+  return kHeaderBytes + align_up((size_t)tiles * 16, 256);
+}
+
+template <typename In, typename Acc, int VE>
+int launch_scan(const In *in, Acc *out, int64_t n, void *ws, size_t ws_bytes, hipStream_t st) {
+  if (n < 0 || n > (1ll << 40)) return n < 0 ? GEAR_HIP_EINVAL : GEAR_HIP_ERANGE;
+  if (n == 0) return 0;
+  if (!in || !out) return GEAR_HIP_EINVAL;
+  if (!ws || ws_bytes < scan_ws_bytes(n) || (reinterpret_cast<uintptr_t>(ws) & 7))
+    return GEAR_HIP_EWORKSPACE;
+  if ((reinterpret_cast<uintptr_t>(in) & (sizeof(In) - 1)) ||
+      (reinterpret_cast<uintptr_t>(out) & 7))
+    return GEAR_HIP_EALIGN;
+  const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
+  uint32_t *ticket = static_cast<uint32_t *>(ws);
+  uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
+  uint64_t *incl = aggr + tiles;
+  const int64_t words = 2 * tiles;
+  scan_init_kernel<<<dim3((unsigned)ceil_div64(words, kBlock)), dim3(kBlock), 0, st>>>(ticket, aggr,
+                                                                                     words);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  scan_kernel<In, Acc, VE><<<dim3((unsigned)tiles), dim3(kBlock), 0, st>>>(in, out, n, ticket, aggr,
+                                                                         incl);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+}  // namespace
+}  // namespace gearhip
+
+using namespace gearhip;
+
+extern "C" size_t gear_hip_scan_workspace_bytes(int64_t n) { return scan_ws_bytes(n); }
+
+extern "C" int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspace,
+                                     size_t workspace_bytes, void *stream) {
+  return launch_scan<float, double, 4>(in, out, n, workspace, workspace_bytes, as_stream(stream));
+}
+
+extern "C" int gear_hip_scan_i64(const int64_t *in, int64_t *out, int64_t n, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+  return launch_scan<int64_t, int64_t, 2>(in, out, n, workspace, workspace_bytes,
+                                          as_stream(stream));
+}
+
+extern "C" size_t gear_hip_sum_workspace_bytes(int64_t n) {
+  (void)n;
+  return kSumMaxBlocks * sizeof(double);
+}
+
+extern "C" int gear_hip_sum_f32(const float *in, int64_t n, float *out, double *out_f64,
+                                void *workspace, size_t workspace_bytes, void *stream) {
+  if (n < 0 || (!out && !out_f64)) return GEAR_HIP_EINVAL;
+  if (n > 0 && !in) return GEAR_HIP_EINVAL;
+  if (!workspace || workspace_bytes < kSumMaxBlocks * sizeof(double)) return GEAR_HIP_EWORKSPACE;
+  if (reinterpret_cast<uintptr_t>(in) & 3) return GEAR_HIP_EALIGN;
+  int64_t blocks = ceil_div64(n, (int64_t)kBlock * 16);
+  if (blocks < 1) blocks = 1;
+  if (blocks > kSumMaxBlocks) blocks = kSumMaxBlocks;
+  double *partial = static_cast<double *>(workspace);
+  hipStream_t st = as_stream(stream);
+  sum_partial_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(in, n, partial);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  sum_final_kernel<<<dim3(1), dim3(kBlock), 0, st>>>(partial, (int)blocks, out, out_f64);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}

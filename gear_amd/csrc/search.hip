@@ -1,0 +1,145 @@
+// Batched upper_bound of draws in an inclusive prefix array (+ importance weights), gfx950.
+//
+// One thread per draw.  The first levels of the binary search touch the same few prefix entries
+// for every draw, so they are served by the caches; the search is latency-bound
+// (log2(n) dependent loads), which is why all draws of a batch run concurrently.
+#include <math.h>
+
+#include "wave.hpp"
+
+namespace gearhip {
+namespace {
+
+constexpr int kBlock = 256;
+
+template <typename T>
+__device__ __forceinline__ int64_t upper_bound_dev(const T *__restrict__ p, int64_t n, T t) {
+  int64_t lo = 0, hi = n;  // first index with p[i] > t
+  while (lo < hi) {
+    const int64_t mid = lo + ((hi - lo) >> 1);
+    if (p[mid] <= t)
+      lo = mid + 1;
+    else
+      hi = mid;
+  }
+  return lo;
+}
+
+__global__ __launch_bounds__(kBlock) void search_f64_kernel(
+    const double *__restrict__ prefix, int64_t n, const float *__restrict__ u, int64_t num,
+    int unit, int64_t *__restrict__ idx_out, const float *__restrict__ priorities, double beta,
+    double *__restrict__ wraw, double *__restrict__ block_max) {
+  __shared__ double wmax[kBlock / kWave];
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const double total = prefix[n - 1];
+  double w = 0.0;
+  if (j < num) {
+    const double t = unit ? (double)u[j] * total : (double)u[j];
+    int64_t i = upper_bound_dev<double>(prefix, n, t);
+    if (i > n - 1) i = n - 1;
+    idx_out[j] = i;
+    if (priorities != nullptr) {
+      w = pow((double)n * (double)priorities[i] / total, -beta);
+      wraw[j] = w;
+    }
+  }
+  if (priorities != nullptr) {
+    // block maximum of the raw weights (weights are positive, padding lanes hold 0)
+    double m = w;
+    for (int off = 32; off > 0; off >>= 1) m = fmax(m, __shfl_xor(m, off, kWave));
+    if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0)
+      block_max[blockIdx.x] = fmax(fmax(wmax[0], wmax[1]), fmax(wmax[2], wmax[3]));
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void normalise_kernel(const double *__restrict__ wraw,
+                                                           const double *__restrict__ block_max,
+                                                           int nblocks, int64_t num,
+                                                           float *__restrict__ out) {
+  __shared__ double wmax[kBlock / kWave];
+  double m = 0.0;
+  for (int i = threadIdx.x; i < nblocks; i += kBlock) m = fmax(m, block_max[i]);
+  for (int off = 32; off > 0; off >>= 1) m = fmax(m, __shfl_xor(m, off, kWave));
+  if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = m;
+  __syncthreads();
+  m = fmax(fmax(wmax[0], wmax[1]), fmax(wmax[2], wmax[3]));
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j < num) out[j] = (float)(wraw[j] / m);
+}
+
+__global__ __launch_bounds__(kBlock) void search_i64_kernel(const int64_t *__restrict__ prefix,
+                                                            int64_t n, const void *u, int64_t num,
+                                                            int unit,
+                                                            int64_t *__restrict__ idx_out) {
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j >= num) return;
+  const int64_t total = prefix[n - 1];
+  int64_t t;
+  if (unit)
+    t = (int64_t)floor(static_cast<const double *>(u)[j] * (double)total);
+  else
+    t = static_cast<const int64_t *>(u)[j];
+  int64_t i = upper_bound_dev<int64_t>(prefix, n, t);
+  if (i > n - 1) i = n - 1;
+  idx_out[j] = i;
+}
+
+size_t search_ws_bytes(int64_t num) {
+  if (num <= 0) return 256;
+  const int64_t blocks = ceil_div64(num, kBlock);
+  return align_up((size_t)num * 8, 256) + align_up((size_t)blocks * 8, 256);
+}
+
+}  // namespace
+}  // namespace gearhip
+
+using namespace gearhip;
+
+extern "C" size_t gear_hip_search_workspace_bytes(int64_t num) { return search_ws_bytes(num); }
+
+extern "C" int gear_hip_upper_bound_f64(const double *prefix, int64_t n, const float *u,
+                                        int64_t num, int unit_uniforms, int64_t *idx_out,
+                                        const float *priorities, double beta, float *weights_out,
+                                        void *workspace, size_t workspace_bytes, void *stream) {
+  if (n < 0 || num < 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (n == 0 || !prefix || !u || !idx_out) return GEAR_HIP_EINVAL;
+  if ((priorities == nullptr) != (weights_out == nullptr)) return GEAR_HIP_EINVAL;
+  const int64_t blocks = ceil_div64(num, kBlock);
+  if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  double *wraw = nullptr, *bmax = nullptr;
+  if (priorities) {
+    if (!workspace || workspace_bytes < search_ws_bytes(num) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 7))
+      return GEAR_HIP_EWORKSPACE;
+    wraw = static_cast<double *>(workspace);
+    bmax = reinterpret_cast<double *>(static_cast<char *>(workspace) +
+                                      align_up((size_t)num * 8, 256));
+  }
+  hipStream_t st = as_stream(stream);
+  search_f64_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(
+      prefix, n, u, num, unit_uniforms ? 1 : 0, idx_out, priorities, beta, wraw, bmax);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  if (priorities) {
+    normalise_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(wraw, bmax, (int)blocks, num,
+                                                                     weights_out);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  }
+  return 0;
+}
+
+extern "C" int gear_hip_upper_bound_i64(const int64_t *prefix, int64_t n, const void *u,
+                                        int64_t num, int unit_uniforms, int64_t *idx_out,
+                                        void *stream) {
+  if (n < 0 || num < 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (n == 0 || !prefix || !u || !idx_out) return GEAR_HIP_EINVAL;
+  const int64_t blocks = ceil_div64(num, kBlock);
+  if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  search_i64_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream)>>>(
+      prefix, n, u, num, unit_uniforms ? 1 : 0, idx_out);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}

@@ -1,0 +1,288 @@
+"""Tensor-level entry points over the C ABI (include/gear_hip.h).
+
+torch tensors are used for what they are here: handles to device memory plus the current HIP
+stream.  All arithmetic happens in libgearhip.so; nothing in this module computes on tensors and
+nothing falls back to torch or to the CPU.
+"""
+import ctypes
+
+import torch
+
+from . import _cabi
+from ._cabi import ColumnDesc, call, load
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _need(t, dtype, name, device=True):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a torch.Tensor" % name)
+    if t.dtype != dtype:
+        raise TypeError("%s must have dtype %s, got %s" % (name, dtype, t.dtype))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    if device and not t.is_cuda:
+        raise ValueError("%s must live on the GPU" % name)
+    return t
+
+
+def _src_ptr(src):
+    """Table base: an int address (MemoryPtr-style), or a tensor (device, or pinned host)."""
+    if isinstance(src, int):
+        return ctypes.c_void_p(src)
+    if isinstance(src, torch.Tensor):
+        return ctypes.c_void_p(src.data_ptr())
+    if hasattr(src, "address"):
+        return ctypes.c_void_p(int(src.address))
+    raise TypeError("unsupported table source %r" % type(src))
+
+
+class _Workspace:
+    """Per-device scratch tensors, grown on demand and reused (no allocation in steady state)."""
+
+    def __init__(self):
+        self._bufs = {}
+
+    def get(self, tag, nbytes, device):
+        key = (tag, device)
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+            self._bufs[key] = buf
+        return buf
+
+
+_ws = _Workspace()
+
+
+def set_device(device_id):
+    call("gear_hip_set_device", int(device_id))
+
+
+def subcopy(src, dst, idxs, tss, lens, *, pad_head, ofst, span, traj_stride, step_bytes,
+            col_base, zero_fill=True, mask_out=None, dst_stride=None):
+    """One column of windows -> dst[num, span, ...]; see gear_hip_subcopy."""
+    _need(idxs, torch.int64, "idxs")
+    _need(tss, torch.int64, "tss")
+    _need(lens, torch.int64, "lens")
+    num = idxs.numel()
+    if tss.numel() != num or lens.numel() != num:
+        raise ValueError("idxs, tss and lens must have the same number of elements")
+    if not dst.is_cuda or not dst.is_contiguous():
+        raise ValueError("dst must be a contiguous GPU tensor")
+    if dst_stride is None:
+        dst_stride = span * step_bytes
+    if dst.numel() * dst.element_size() < num * dst_stride:
+        raise ValueError("dst is smaller than num * dst_stride bytes")
+    if mask_out is not None:
+        _need(mask_out, torch.uint8, "mask_out")
+        if mask_out.numel() < num * span:
+            raise ValueError("mask_out is smaller than num * span")
+    call("gear_hip_subcopy", _src_ptr(src), _ptr(dst), num, _ptr(idxs), _ptr(tss), _ptr(lens),
+         int(bool(pad_head)), int(ofst), int(span), int(traj_stride), int(step_bytes),
+         int(col_base), int(dst_stride), int(bool(zero_fill)), _ptr(mask_out), _stream())
+    return dst
+
+
+def subcopy_multi(src, idxs, tss, lens, traj_stride, columns):
+    """All columns of one batch in one launch.
+
+    columns: list of dicts with keys dst, ofst, span, step_bytes, col_base, pad_head and
+    optionally zero_fill (default True), mask_out, dst_stride.
+    """
+    _need(idxs, torch.int64, "idxs")
+    _need(tss, torch.int64, "tss")
+    _need(lens, torch.int64, "lens")
+    num = idxs.numel()
+    n = len(columns)
+    if n > _cabi.MAX_COLUMNS:
+        raise ValueError("at most %d columns per launch" % _cabi.MAX_COLUMNS)
+    descs = (ColumnDesc * max(n, 1))()
+    for i, c in enumerate(columns):
+        dst = c["dst"]
+        stride = c.get("dst_stride", c["span"] * c["step_bytes"])
+        if not dst.is_cuda or not dst.is_contiguous():
+            raise ValueError("column %d: dst must be a contiguous GPU tensor" % i)
+        if dst.numel() * dst.element_size() < num * stride:
+            raise ValueError("column %d: dst is smaller than num * dst_stride bytes" % i)
+        m = c.get("mask_out")
+        if m is not None and m.numel() < num * c["span"]:
+            raise ValueError("column %d: mask_out is smaller than num * span" % i)
+        descs[i].dst = dst.data_ptr()
+        descs[i].mask_out = m.data_ptr() if m is not None else None
+        descs[i].ofst = int(c["ofst"])
+        descs[i].span = int(c["span"])
+        descs[i].step_bytes = int(c["step_bytes"])
+        descs[i].col_base = int(c["col_base"])
+        descs[i].dst_stride = int(stride)
+        descs[i].pad_head = int(bool(c["pad_head"]))
+        descs[i].zero_fill = int(bool(c.get("zero_fill", True)))
+    call("gear_hip_subcopy_multi", _src_ptr(src), num, _ptr(idxs), _ptr(tss), _ptr(lens),
+         int(traj_stride), descs, n, _stream())
+
+
+def vcopy(src, dst, src_offsets, dst_offsets, strides, max_stride):
+    _need(src_offsets, torch.int64, "src_offsets")
+    _need(dst_offsets, torch.int64, "dst_offsets")
+    _need(strides, torch.int64, "strides")
+    num = min(src_offsets.numel(), dst_offsets.numel(), strides.numel())
+    call("gear_hip_vcopy", _src_ptr(src), _ptr(dst), num, _ptr(src_offsets), _ptr(dst_offsets),
+         _ptr(strides), int(max_stride), _stream())
+    return dst
+
+
+def copy(src, dst, src_offsets, dst_offsets, stride):
+    _need(src_offsets, torch.int64, "src_offsets")
+    _need(dst_offsets, torch.int64, "dst_offsets")
+    num = min(src_offsets.numel(), dst_offsets.numel())
+    call("gear_hip_copy", _src_ptr(src), _ptr(dst), num, _ptr(src_offsets), _ptr(dst_offsets),
+         int(stride), _stream())
+    return dst
+
+
+def sub(idxs, tss, lens, *, pad_head, ofst, span, traj_stride, step_bytes, col_base,
+        src_offsets=None, dst_offsets=None, copy_lens=None):
+    _need(idxs, torch.int64, "idxs")
+    _need(tss, torch.int64, "tss")
+    _need(lens, torch.int64, "lens")
+    num = idxs.numel()
+    outs = []
+    for t in (src_offsets, dst_offsets, copy_lens):
+        outs.append(t if t is not None else torch.empty(num, dtype=torch.int64,
+                                                        device=idxs.device))
+    call("gear_hip_sub", num, _ptr(idxs), _ptr(tss), _ptr(lens), int(bool(pad_head)), int(ofst),
+         int(span), int(traj_stride), int(step_bytes), int(col_base), _ptr(outs[0]),
+         _ptr(outs[1]), _ptr(outs[2]), _stream())
+    return outs[0], outs[1], outs[2], span * step_bytes
+
+
+def prefix_sum(priorities, out=None):
+    """fp32[n] -> inclusive fp64 prefix[n] (gear_hip_scan_f32_f64)."""
+    _need(priorities, torch.float32, "priorities")
+    n = priorities.numel()
+    if out is None:
+        out = torch.empty(n, dtype=torch.float64, device=priorities.device)
+    else:
+        _need(out, torch.float64, "out")
+        if out.numel() < n:
+            raise ValueError("out is too small")
+    nbytes = load().gear_hip_scan_workspace_bytes(n)
+    ws = _ws.get("scan", nbytes, priorities.device)
+    call("gear_hip_scan_f32_f64", _ptr(priorities), _ptr(out), n, _ptr(ws), ws.numel(), _stream())
+    return out
+
+
+def prefix_sum_i64(weights, out=None):
+    _need(weights, torch.int64, "weights")
+    n = weights.numel()
+    if out is None:
+        out = torch.empty(n, dtype=torch.int64, device=weights.device)
+    else:
+        _need(out, torch.int64, "out")
+    nbytes = load().gear_hip_scan_workspace_bytes(n)
+    ws = _ws.get("scan", nbytes, weights.device)
+    call("gear_hip_scan_i64", _ptr(weights), _ptr(out), n, _ptr(ws), ws.numel(), _stream())
+    return out
+
+
+def sum_f32(values, out=None, out_f64=None):
+    _need(values, torch.float32, "values")
+    n = values.numel()
+    if out is None:
+        out = torch.empty(1, dtype=torch.float32, device=values.device)
+    nbytes = load().gear_hip_sum_workspace_bytes(n)
+    ws = _ws.get("sum", nbytes, values.device)
+    call("gear_hip_sum_f32", _ptr(values), n, _ptr(out), _ptr(out_f64), _ptr(ws), ws.numel(),
+         _stream())
+    return out
+
+
+def upper_bound(prefix, u, *, unit_uniforms=False, idx_out=None, priorities=None, beta=0.4,
+                weights_out=None):
+    """Batched search of draws in an fp64 prefix array; optionally importance weights."""
+    _need(prefix, torch.float64, "prefix")
+    _need(u, torch.float32, "u")
+    num = u.numel()
+    if idx_out is None:
+        idx_out = torch.empty(num, dtype=torch.int64, device=u.device)
+    else:
+        _need(idx_out, torch.int64, "idx_out")
+    ws = None
+    if priorities is not None:
+        _need(priorities, torch.float32, "priorities")
+        if priorities.numel() != prefix.numel():
+            raise ValueError("priorities and prefix differ in length")
+        if weights_out is None:
+            weights_out = torch.empty(num, dtype=torch.float32, device=u.device)
+        nbytes = load().gear_hip_search_workspace_bytes(num)
+        ws = _ws.get("search", nbytes, u.device)
+    call("gear_hip_upper_bound_f64", _ptr(prefix), prefix.numel(), _ptr(u), num,
+         int(bool(unit_uniforms)), _ptr(idx_out), _ptr(priorities), float(beta),
+         _ptr(weights_out) if priorities is not None else None, _ptr(ws),
+         ws.numel() if ws is not None else 0, _stream())
+    if priorities is not None:
+        return idx_out, weights_out
+    return idx_out
+
+
+def upper_bound_i64(prefix, u, *, unit_uniforms=True, idx_out=None):
+    _need(prefix, torch.int64, "prefix")
+    _need(u, torch.float64 if unit_uniforms else torch.int64, "u")
+    num = u.numel()
+    if idx_out is None:
+        idx_out = torch.empty(num, dtype=torch.int64, device=u.device)
+    call("gear_hip_upper_bound_i64", _ptr(prefix), prefix.numel(), _ptr(u), num,
+         int(bool(unit_uniforms)), _ptr(idx_out), _stream())
+    return idx_out
+
+
+def sort_i64(keys, vals=None, key_bits=63):
+    _need(keys, torch.int64, "keys")
+    num = keys.numel()
+    keys_out = torch.empty_like(keys)
+    vals_out = None
+    if vals is not None:
+        _need(vals, torch.int64, "vals")
+        vals_out = torch.empty_like(vals)
+    nbytes = load().gear_hip_sort_workspace_bytes(num)
+    ws = _ws.get("sort", nbytes, keys.device)
+    call("gear_hip_sort_i64", _ptr(keys), _ptr(keys_out), _ptr(vals), _ptr(vals_out), num,
+         int(key_bits), _ptr(ws), ws.numel(), _stream())
+    return (keys_out, vals_out) if vals is not None else keys_out
+
+
+def topk(priorities, k, *, sorted_by_value=True, want_values=True):
+    _need(priorities, torch.float32, "priorities")
+    n = priorities.numel()
+    idx = torch.empty(k, dtype=torch.int64, device=priorities.device)
+    vals = torch.empty(k, dtype=torch.float32, device=priorities.device) if want_values else None
+    nbytes = load().gear_hip_topk_workspace_bytes(n, k)
+    ws = _ws.get("topk", nbytes, priorities.device)
+    call("gear_hip_topk_f32", _ptr(priorities), n, int(k), int(bool(sorted_by_value)), _ptr(vals),
+         _ptr(idx), _ptr(ws), ws.numel(), _stream())
+    return vals, idx
+
+
+def scatter(weights, idx, values, *, unique_indices=False):
+    """weights[idx[j]] = values[j]; duplicates: last one wins."""
+    _need(weights, torch.float32, "weights")
+    _need(idx, torch.int64, "idx")
+    _need(values, torch.float32, "values")
+    num = idx.numel()
+    if values.numel() != num:
+        raise ValueError("idx and values differ in length")
+    ws = None
+    if not unique_indices:
+        nbytes = load().gear_hip_scatter_workspace_bytes(num)
+        ws = _ws.get("scatter", nbytes, weights.device)
+    call("gear_hip_scatter_f32", _ptr(weights), weights.numel(), _ptr(idx), _ptr(values), num,
+         int(bool(unique_indices)), _ptr(ws), ws.numel() if ws is not None else 0, _stream())
+    return weights

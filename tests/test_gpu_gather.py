@@ -1,0 +1,287 @@
+"""GPU parity of the window gather (gear_hip_subcopy / _multi / vcopy / copy / sub) through the
+C ABI, against the CPU oracle and an independent numpy gather, bit-exact."""
+import numpy as np
+import pytest
+
+from conftest import announce
+from helpers import Schema, fill_random, numpy_window_gather
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+CFG1 = [("obs", "float32", (17,)), ("action", "float32", (6,)), ("reward", "float32", ()),
+        ("done", "uint8", ())]
+CFG3 = [("obs", "float32", (17,)), ("action", "float32", (6,)), ("reward", "float32", ()),
+        ("rtg", "float32", ()), ("timestep", "int32", ())]
+CFG4 = [("obs", "uint8", (4, 84, 84)), ("action", "int32", ()), ("reward", "float32", ()),
+        ("done", "uint8", ())]
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _run_subcopy(ops, schema, table_dev, c, idxs, tss, lens, ofst, span, pad_head,
+                 zero_fill=True, want_mask=True, prefill=0xAB):
+    sb = schema.step_bytes[c]
+    n = len(idxs)
+    dst = torch.full((n, span * sb), prefill, dtype=torch.uint8, device="cuda")
+    mask = torch.full((n, span), 7, dtype=torch.uint8, device="cuda") if want_mask else None
+    ops.subcopy(table_dev, dst, _dev(idxs), _dev(tss), _dev(lens), pad_head=pad_head, ofst=ofst,
+                span=span, traj_stride=schema.traj_stride, step_bytes=sb,
+                col_base=schema.col_base(c), zero_fill=zero_fill, mask_out=mask)
+    torch.cuda.synchronize()
+    return dst.cpu().numpy(), (mask.cpu().numpy() if want_mask else None)
+
+
+def test_config1_full_trajectories(oracle):
+    """BASELINE config 1 at full size: 4096 x 64 table, 256 uniformly drawn trajectories."""
+    from gear_amd import ops
+    schema = Schema(CFG1, T=64, capacity=4096)
+    table = fill_random(schema, 1001)
+    rng = np.random.default_rng(1001)
+    idxs = (rng.integers(0, 2**32, size=256, dtype=np.uint64) % 4096).astype(np.int64)
+    tss = np.zeros(256, np.int64)
+    lens = np.full(256, 64, np.int64)
+    tdev = _dev(table)
+    for c in range(4):
+        announce("config1 column %d" % c)
+        got, mask = _run_subcopy(ops, schema, tdev, c, idxs, tss, lens, 0, 64, False)
+        exp, emask = oracle.subcopy(table, idxs, tss, lens, False, 0, 64, schema.traj_stride,
+                                    schema.step_bytes[c], schema.col_base(c), want_mask=True)
+        ref, _ = numpy_window_gather(schema, table, c, idxs, tss, lens, 0, 64, False)
+        assert np.array_equal(exp, ref)
+        assert np.array_equal(got, exp)
+        assert np.array_equal(mask, emask)
+
+
+@pytest.mark.parametrize("pad_head", [False, True])
+def test_config3_windows_with_padding(oracle, pad_head):
+    """Config 3 schema (scaled to 1000 trajectories): 20-step windows, variable lengths, starts up
+    to len-1 and before 0 so that head/tail padding and empty windows occur."""
+    from gear_amd import ops
+    schema = Schema(CFG3, T=1000, capacity=1000)
+    table = fill_random(schema, 1003)
+    rng = np.random.default_rng(1003 + int(pad_head))
+    B = 1024
+    idxs = rng.integers(0, 1000, size=B).astype(np.int64)
+    lens = rng.integers(200, 1001, size=B).astype(np.int64)
+    tss = (rng.integers(0, 1 << 30, size=B) % lens).astype(np.int64)
+    tss[:8] = lens[:8] - 1          # one valid step, 19 padded
+    tss[8:16] = lens[8:16]          # starts at len: empty window
+    tss[16:24] = lens[16:24] + 5    # beyond the end
+    tdev = _dev(table)
+    for ofst in (0, -19, -25):
+        for c in range(5):
+            announce("config3 pad_head=%s ofst=%d column %d" % (pad_head, ofst, c))
+            got, mask = _run_subcopy(ops, schema, tdev, c, idxs, tss, lens, ofst, 20, pad_head)
+            exp, emask = oracle.subcopy(table, idxs, tss, lens, pad_head, ofst, 20,
+                                        schema.traj_stride, schema.step_bytes[c],
+                                        schema.col_base(c), want_mask=True)
+            ref, rmask = numpy_window_gather(schema, table, c, idxs, tss, lens, ofst, 20, pad_head)
+            assert np.array_equal(exp, ref) and np.array_equal(emask, rmask)
+            assert np.array_equal(got, exp)
+            assert np.array_equal(mask, emask)
+
+
+def test_config4_scaled_all_columns_and_multi(oracle):
+    """Config 4 schema, 50 trajectories x 100 steps (141 MB): (-29, 30, head) windows with
+    lens = ts + 1, per-column launches and the one-launch multi-column entry point."""
+    from gear_amd import ops
+    schema = Schema(CFG4, T=100, capacity=50)
+    table = fill_random(schema, 1004)
+    rng = np.random.default_rng(1004)
+    B = 96
+    idxs = rng.integers(0, 50, size=B).astype(np.int64)
+    tss = rng.integers(0, 100, size=B).astype(np.int64)
+    tss[:6] = [0, 1, 5, 28, 29, 99]
+    lens = tss + 1
+    tdev = _dev(table)
+    exps = []
+    for c in range(4):
+        announce("config4-scaled column %d" % c)
+        got, mask = _run_subcopy(ops, schema, tdev, c, idxs, tss, lens, -29, 30, True)
+        exp, emask = oracle.subcopy(table, idxs, tss, lens, True, -29, 30, schema.traj_stride,
+                                    schema.step_bytes[c], schema.col_base(c), want_mask=True)
+        if c > 0:  # the obs column is large; numpy cross-check on the small ones
+            ref, _ = numpy_window_gather(schema, table, c, idxs, tss, lens, -29, 30, True)
+            assert np.array_equal(exp, ref)
+        assert np.array_equal(got, exp)
+        assert np.array_equal(mask, emask)
+        exps.append((exp, emask))
+    announce("config4-scaled multi-column launch")
+    dsts = [torch.full((B, 30 * schema.step_bytes[c]), 0xCD, dtype=torch.uint8, device="cuda")
+            for c in range(4)]
+    masks = [torch.full((B, 30), 9, dtype=torch.uint8, device="cuda") for _ in range(4)]
+    cols = [dict(dst=dsts[c], mask_out=masks[c], ofst=-29, span=30,
+                 step_bytes=schema.step_bytes[c], col_base=schema.col_base(c), pad_head=True)
+            for c in range(4)]
+    ops.subcopy_multi(tdev, _dev(idxs), _dev(tss), _dev(lens), schema.traj_stride, cols)
+    torch.cuda.synchronize()
+    for c in range(4):
+        assert np.array_equal(dsts[c].cpu().numpy(), exps[c][0])
+        assert np.array_equal(masks[c].cpu().numpy(), exps[c][1])
+
+
+def test_no_zero_fill_leaves_padding_untouched(oracle):
+    """zero_fill=0 is the reference's contract: only copied bytes are written."""
+    from gear_amd import ops
+    schema = Schema(CFG3, T=64, capacity=64)
+    table = fill_random(schema, 7)
+    rng = np.random.default_rng(7)
+    B = 200
+    idxs = rng.integers(0, 64, size=B).astype(np.int64)
+    lens = rng.integers(1, 65, size=B).astype(np.int64)
+    tss = rng.integers(0, 64, size=B).astype(np.int64)
+    tdev = _dev(table)
+    for pad_head in (False, True):
+        for c in (0, 4):
+            announce("no-zero-fill pad_head=%s column %d" % (pad_head, c))
+            got, _ = _run_subcopy(ops, schema, tdev, c, idxs, tss, lens, -3, 9, pad_head,
+                                  zero_fill=False, want_mask=False, prefill=0xAB)
+            pre = np.full((B, 9 * schema.step_bytes[c]), 0xAB, np.uint8)
+            exp, _ = oracle.subcopy(table, idxs, tss, lens, pad_head, -3, 9, schema.traj_stride,
+                                    schema.step_bytes[c], schema.col_base(c), zero_fill=False,
+                                    dst=pre)
+            assert np.array_equal(got, exp)
+
+
+def test_odd_byte_columns_every_alignment(oracle):
+    """1-, 3- and 7-byte steps: windows start on any byte, dst windows are not 16-byte multiples."""
+    from gear_amd import ops
+    cols = [("a", "uint8", ()), ("b", "uint8", (3,)), ("c", "uint8", (7,)), ("d", "int16", (5,))]
+    schema = Schema(cols, T=37, capacity=29)
+    table = fill_random(schema, 11)
+    rng = np.random.default_rng(11)
+    B = 333
+    idxs = rng.integers(0, 29, size=B).astype(np.int64)
+    lens = rng.integers(0, 38, size=B).astype(np.int64)
+    tss = rng.integers(0, 37, size=B).astype(np.int64)
+    tdev = _dev(table)
+    for span in (1, 5, 30):
+        for pad_head in (False, True):
+            for c in range(4):
+                announce("odd-bytes span=%d pad_head=%s column %d" % (span, pad_head, c))
+                got, mask = _run_subcopy(ops, schema, tdev, c, idxs, tss, lens, -2, span, pad_head)
+                ref, rmask = numpy_window_gather(schema, table, c, idxs, tss, lens, -2, span,
+                                                 pad_head)
+                assert np.array_equal(got, ref)
+                assert np.array_equal(mask, rmask)
+
+
+def test_empty_batch():
+    from gear_amd import ops
+    t = torch.zeros(1024, dtype=torch.uint8, device="cuda")
+    e = torch.zeros(0, dtype=torch.int64, device="cuda")
+    dst = torch.zeros(0, dtype=torch.uint8, device="cuda")
+    announce("empty batch")
+    ops.subcopy(t, dst, e, e, e, pad_head=False, ofst=0, span=4, traj_stride=64, step_bytes=4,
+                col_base=0)
+    ops.vcopy(t, dst, e, e, e, 16)
+    ops.copy(t, dst, e, e, 16)
+    torch.cuda.synchronize()
+
+
+def test_vcopy_copy_and_sub_against_oracle(oracle):
+    """Generic slice gathers with arbitrary byte offsets and lengths (reference: tests/test_sub.py
+    feeds handler.sub output to vcopy); device sub == oracle sub."""
+    from gear_amd import ops
+    rng = np.random.default_rng(21)
+    src = rng.integers(0, 256, size=1 << 20, dtype=np.uint8)
+    sdev = _dev(src)
+    for max_len in (1, 15, 16, 17, 96, 4096, 70001):
+        B = 257
+        lens = rng.integers(0, max_len + 1, size=B).astype(np.int64)
+        lens[0] = max_len
+        so = rng.integers(0, (1 << 20) - max_len, size=B).astype(np.int64)
+        do = np.zeros(B, np.int64)
+        do[1:] = np.cumsum(lens[:-1] + rng.integers(0, 5, size=B - 1))
+        total = int(do[-1] + lens[-1]) + 8
+        announce("vcopy max_len=%d" % max_len)
+        dst = torch.full((total,), 0x5A, dtype=torch.uint8, device="cuda")
+        ops.vcopy(sdev, dst, _dev(so), _dev(do), _dev(lens), max_len)
+        torch.cuda.synchronize()
+        exp = oracle.vcopy(src, np.full(total, 0x5A, np.uint8), so, do, lens)
+        assert np.array_equal(dst.cpu().numpy(), exp)
+        announce("copy stride=%d" % max_len)
+        do2 = np.arange(B, dtype=np.int64) * (max_len + 3)
+        dst2 = torch.full((B * (max_len + 3),), 0x5A, dtype=torch.uint8, device="cuda")
+        ops.copy(sdev, dst2, _dev(so), _dev(do2), max_len)
+        torch.cuda.synchronize()
+        exp2 = oracle.copy(src, np.full(B * (max_len + 3), 0x5A, np.uint8), so, do2, max_len)
+        assert np.array_equal(dst2.cpu().numpy(), exp2)
+
+    announce("device sub vs oracle sub")
+    B = 1000
+    idxs = rng.integers(0, 5000, size=B).astype(np.int64)
+    lens = rng.integers(0, 100, size=B).astype(np.int64)
+    tss = rng.integers(0, 100, size=B).astype(np.int64)
+    for pad_head in (False, True):
+        for ofst in (-7, 0, 3):
+            so, do, cl, exp_len = ops.sub(_dev(idxs), _dev(tss), _dev(lens), pad_head=pad_head,
+                                          ofst=ofst, span=10, traj_stride=9600, step_bytes=96,
+                                          col_base=1200)
+            torch.cuda.synchronize()
+            eso, edo, ecl, eexp = oracle.sub(idxs, tss, lens, pad_head, ofst, 10, 9600, 96, 1200)
+            assert exp_len == eexp
+            assert np.array_equal(so.cpu().numpy(), eso)
+            assert np.array_equal(do.cpu().numpy(), edo)
+            assert np.array_equal(cl.cpu().numpy(), ecl)
+
+
+def test_reference_copy_test_shape():
+    """tests/test_copy.py of the reference: pinned ones[32,100,4,3,2] fp32, one 960-byte slice
+    through copy_debug (vary-stride gather) -> everything non-zero; here from pinned host memory
+    read in place by the GPU."""
+    from gear_amd import ops
+    data = torch.ones((32, 100, 4, 3, 2), dtype=torch.float32, pin_memory=True)
+    copied = torch.zeros((10, 4, 3, 2), dtype=torch.float32, device="cuda")
+    zero = torch.zeros(1, dtype=torch.int64, device="cuda")
+    stride = torch.full((1,), copied.numel() * 4, dtype=torch.int64, device="cuda")
+    announce("reference test_copy shape from pinned host memory")
+    ops.vcopy(data, copied, zero, zero, stride, copied.numel() * 4)
+    torch.cuda.synchronize()
+    assert bool(torch.all(copied == 1.0))
+
+
+def test_config4_full_size_property():
+    """Config 4 at full size (28.2 GB table in HBM, 2048 x 30-step windows): checked on the
+    device against torch indexing of the same table, window by window, bit-exact."""
+    from gear_amd import ops
+    schema = Schema(CFG4, T=1000, capacity=1000)
+    free, _ = torch.cuda.mem_get_info()
+    if free < schema.nbytes + (8 << 30):
+        pytest.skip("not enough free HBM for the 28.2 GB table")
+    announce("config4 full size: building table")
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1004)
+    table = torch.empty(schema.nbytes, dtype=torch.uint8, device="cuda")
+    step = 1 << 30
+    for o in range(0, schema.nbytes, step):
+        n = min(step, schema.nbytes - o)
+        table[o:o + n] = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda", generator=g)
+    rng = np.random.default_rng(1004)
+    B = 2048
+    flat = rng.integers(0, 1000 * 1000, size=B)
+    flat[:4] = [0, 5, 28, 999999]
+    idxs = (flat // 1000).astype(np.int64)
+    tss = (flat % 1000).astype(np.int64)
+    lens = tss + 1
+    di, dt, dl = _dev(idxs), _dev(tss), _dev(lens)
+    dsts = [torch.empty((B, 30 * schema.step_bytes[c]), dtype=torch.uint8, device="cuda")
+            for c in range(4)]
+    cols = [dict(dst=dsts[c], ofst=-29, span=30, step_bytes=schema.step_bytes[c],
+                 col_base=schema.col_base(c), pad_head=True) for c in range(4)]
+    announce("config4 full size: multi-column gather")
+    ops.subcopy_multi(table, di, dt, dl, schema.traj_stride, cols)
+    torch.cuda.synchronize()
+    announce("config4 full size: checking")
+    for c in range(4):
+        sb = schema.step_bytes[c]
+        for gidx in range(B):
+            start = max(int(tss[gidx]) - 29, 0)
+            steps = int(tss[gidx]) + 1 - start
+            a = int(idxs[gidx]) * schema.traj_stride + schema.col_base(c) + start * sb
+            row = dsts[c][gidx]
+            assert torch.equal(row[(30 - steps) * sb:], table[a:a + steps * sb])
+            assert int(row[:(30 - steps) * sb].max().item() if steps < 30 else 0) == 0

@@ -1,0 +1,112 @@
+"""GPU parity of the sort / top-k / priority-update path through the C ABI vs the CPU oracle."""
+import numpy as np
+import pytest
+
+from conftest import announce
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _check_topk(oracle, ops, w, k, label):
+    announce("topk %s n=%d k=%d" % (label, len(w), k))
+    dw = _dev(w)
+    vals, idx = ops.topk(dw, k, sorted_by_value=True)
+    uvals, uidx = ops.topk(dw, k, sorted_by_value=False)
+    torch.cuda.synchronize()
+    evals, eidx = oracle.topk_f32(w, k, True)
+    assert np.array_equal(idx.cpu().numpy(), eidx)
+    assert np.array_equal(vals.cpu().numpy().view(np.uint32), evals.view(np.uint32))
+    _, euidx = oracle.topk_f32(w, k, False)
+    assert np.array_equal(uidx.cpu().numpy(), euidx)
+    assert np.array_equal(uvals.cpu().numpy().view(np.uint32), w[euidx].view(np.uint32))
+    # independent statement: stable descending argsort
+    ref = np.argsort(-w.astype(np.float64), kind="stable")[:k]
+    assert np.array_equal(eidx, ref)
+
+
+def test_topk_cases(oracle):
+    from gear_amd import ops
+    rng = np.random.default_rng(31)
+    ln = lambda n: (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    _check_topk(oracle, ops, ln(1000), 1, "lognormal")
+    _check_topk(oracle, ops, ln(1000), 1000, "k == n")
+    _check_topk(oracle, ops, ln(5000), 4999, "k == n-1")
+    _check_topk(oracle, ops, ln(4097), 33, "tile + 1")
+    _check_topk(oracle, ops, np.full(10000, 2.5, np.float32), 777, "all equal")
+    _check_topk(oracle, ops, rng.integers(0, 4, size=100_000).astype(np.float32), 30_000,
+                "four distinct values")
+    _check_topk(oracle, ops, rng.integers(0, 1000, size=1_000_000).astype(np.float32), 65_536,
+                "many ties at the threshold")
+    special = ln(20_000)
+    special[:6] = [0.0, np.inf, np.float32(1e-45), np.float32(1e-40), 3.4e38, 0.0]
+    _check_topk(oracle, ops, special, 19_998, "zeros / inf / denormals")
+    mixed = rng.normal(size=50_000).astype(np.float32)  # negative values order correctly too
+    _check_topk(oracle, ops, mixed, 12_345, "signed")
+
+
+def test_topk_config5_size(oracle):
+    """Config 5's maintenance step at full size: top-65 536 of 10 000 000 lognormal^0.6."""
+    from gear_amd import ops
+    rng = np.random.default_rng(1005)
+    w = (rng.lognormal(0, 1, size=10_000_000) ** 0.6).astype(np.float32)
+    _check_topk(oracle, ops, w, 65_536, "config5")
+
+
+def test_sort_i64(oracle):
+    from gear_amd import ops
+    rng = np.random.default_rng(41)
+    for n, bits in ((1, 1), (2, 8), (255, 9), (256, 20), (1025, 20), (2048, 24), (4096, 31),
+                    (65_536, 40), (300_001, 63)):
+        keys = rng.integers(0, 1 << min(bits, 62), size=n).astype(np.int64)
+        keys[rng.integers(0, n, size=max(n // 3, 1))] = keys[0]  # duplicates: stability matters
+        vals = rng.integers(-2**62, 2**62, size=n).astype(np.int64)
+        announce("sort n=%d bits=%d" % (n, bits))
+        ko, vo = ops.sort_i64(_dev(keys), _dev(vals), key_bits=bits)
+        k2 = ops.sort_i64(_dev(keys), key_bits=bits)
+        torch.cuda.synchronize()
+        ek, ev = oracle.sort_i64(keys, vals)
+        assert np.array_equal(ko.cpu().numpy(), ek)
+        assert np.array_equal(vo.cpu().numpy(), ev)
+        assert np.array_equal(k2.cpu().numpy(), ek)
+        order = np.argsort(keys, kind="stable")
+        assert np.array_equal(ek, keys[order]) and np.array_equal(ev, vals[order])
+
+
+def test_scatter_unique_and_duplicates(oracle):
+    from gear_amd import ops
+    rng = np.random.default_rng(51)
+    n = 1_000_000
+    w0 = rng.random(n, dtype=np.float32)
+    # unique indices: a seeded permutation prefix
+    idx = rng.permutation(n)[:65_536].astype(np.int64)
+    v = rng.random(65_536, dtype=np.float32)
+    for unique in (True, False):
+        announce("scatter unique input, unique_indices=%s" % unique)
+        dw = _dev(w0)
+        ops.scatter(dw, _dev(idx), _dev(v), unique_indices=unique)
+        torch.cuda.synchronize()
+        exp = oracle.scatter_f32(w0.copy(), idx, v)
+        ref = w0.copy()
+        ref[idx] = v
+        assert np.array_equal(exp, ref)
+        assert np.array_equal(dw.cpu().numpy(), exp)
+    # duplicates (each index about 8 times) + out-of-range entries: last write wins
+    idx = rng.integers(0, 8192, size=65_536).astype(np.int64)
+    idx[::1000] = -1
+    idx[1::1000] = n + 5
+    announce("scatter with duplicates")
+    dw = _dev(w0)
+    ops.scatter(dw, _dev(idx), _dev(v), unique_indices=False)
+    torch.cuda.synchronize()
+    exp = oracle.scatter_f32(w0.copy(), idx, v)
+    ref = w0.copy()
+    for j in range(len(idx)):          # brute-force "last wins"
+        if 0 <= idx[j] < n:
+            ref[idx[j]] = v[j]
+    assert np.array_equal(exp, ref)
+    assert np.array_equal(dw.cpu().numpy(), exp)
