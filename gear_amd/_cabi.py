@@ -47,6 +47,8 @@ SIGNATURES = {
     "gear_hip_copy": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_i64, c_void_p]),
     "gear_hip_sub": (c_int, [c_i64, c_void_p, c_void_p, c_void_p, c_int, c_i64, c_i64, c_i64,
                              c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "gear_hip_split_step_index": (c_int, [c_void_p, c_i64, c_i64, c_i64, c_void_p, c_void_p,
+                                          c_void_p, c_void_p]),
     "gear_hip_scan_workspace_bytes": (c_size_t, [c_i64]),
     "gear_hip_scan_f32_f64": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_size_t, c_void_p]),
     "gear_hip_scan_i64": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_size_t, c_void_p]),

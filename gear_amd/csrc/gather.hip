@@ -251,6 +251,23 @@ __global__ __launch_bounds__(kBlock) void sub_kernel(int64_t num, const int64_t 
   dst_offsets[i] = expected * i + (pad_head ? expected - copy_len : 0);
 }
 
+// flat step index -> (trajectory, timestep, length = timestep + 1)
+__global__ __launch_bounds__(kBlock) void split_kernel(const int64_t *__restrict__ flat,
+                                                       int64_t num, int64_t T, int64_t modulo,
+                                                       int64_t *__restrict__ idxs,
+                                                       int64_t *__restrict__ tss,
+                                                       int64_t *__restrict__ lens) {
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j >= num) return;
+  int64_t f = flat[j];
+  if (modulo > 0) f %= modulo;
+  const int64_t traj = f / T;
+  const int64_t ts = f - traj * T;
+  idxs[j] = traj;
+  tss[j] = ts;
+  if (lens) lens[j] = ts + 1;
+}
+
 struct Shape {
   int tg_shift;
   int64_t cps;
@@ -448,6 +465,20 @@ extern "C" int gear_hip_sub(int64_t num, const int64_t *idxs, const int64_t *tss
   sub_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream)>>>(
       num, idxs, tss, lens, pad_head ? 1 : 0, ofst, span, traj_stride, step_bytes, col_base,
       src_offsets, dst_offsets, copy_lens);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+extern "C" int gear_hip_split_step_index(const int64_t *flat, int64_t num, int64_t trajectory_length,
+                                         int64_t modulo, int64_t *idxs, int64_t *tss,
+                                         int64_t *lens, void *stream) {
+  if (num < 0 || trajectory_length <= 0 || modulo < 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (!flat || !idxs || !tss) return GEAR_HIP_EINVAL;
+  const int64_t blocks = ceil_div64(num, kBlock);
+  if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  split_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream)>>>(
+      flat, num, trajectory_length, modulo, idxs, tss, lens);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

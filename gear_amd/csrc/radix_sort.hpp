@@ -38,7 +38,8 @@ inline size_t hist_bytes(int64_t num) {
 
 template <typename K>
 __global__ __launch_bounds__(kBlock) void hist_kernel(const K *__restrict__ keys, int64_t num,
-                                                      int shift, int rounds, int64_t ntiles,
+                                                      int shift, uint32_t dmask, int rounds,
+                                                      int64_t ntiles,
                                                       uint32_t *__restrict__ hist) {
   __shared__ uint32_t h[kBins];
   const int tid = threadIdx.x;
@@ -47,7 +48,7 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const K *__restrict__ keys
   const int64_t base = (int64_t)blockIdx.x * kBlock * rounds;
   for (int r = 0; r < rounds; ++r) {
     const int64_t i = base + (int64_t)r * kBlock + tid;
-    if (i < num) atomicAdd(&h[(uint32_t)(keys[i] >> shift) & 255u], 1u);
+    if (i < num) atomicAdd(&h[(uint32_t)(keys[i] >> shift) & dmask], 1u);
   }
   __syncthreads();
   hist[(int64_t)tid * ntiles + blockIdx.x] = h[tid];
@@ -83,7 +84,8 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(const K *__restrict__ k
                                                          const V *__restrict__ vin,
                                                          K *__restrict__ kout,
                                                          V *__restrict__ vout, int64_t num,
-                                                         int shift, int rounds, int64_t ntiles,
+                                                         int shift, uint32_t dmask, int rounds,
+                                                         int64_t ntiles,
                                                          const uint32_t *__restrict__ offsets) {
   __shared__ uint32_t base[kBins];
   __shared__ uint32_t wcnt[kWaves][kBins];
@@ -98,7 +100,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(const K *__restrict__ k
     const int64_t i = tile0 + (int64_t)r * kBlock + tid;
     const bool valid = i < num;
     const K key = valid ? kin[i] : (K)0;
-    const uint32_t d = (uint32_t)(key >> shift) & 255u;
+    const uint32_t d = (uint32_t)(key >> shift) & dmask;
     uint64_t peers = wave_ballot(valid);
 #pragma unroll
     for (int b = 0; b < 8; ++b) {
@@ -129,6 +131,96 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(const K *__restrict__ k
   }
 }
 
+// ---- one-workgroup sort for small batches (a sampled batch of indices) --------------------------
+// Up to kSmallMax keys stay in registers (4 per thread, element e = r*1024 + tid) and move
+// through LDS once per 4-bit digit: ballots rank equal digits inside a wave, a 16 x 64 table of
+// (digit, round*16+wave) counts is scanned by the 1024 threads, one counter each.  The payload is
+// carried as the element's original position and applied with one global gather at the end.
+constexpr int kSmallBlock = 1024;
+constexpr int kSmallRounds = 4;
+constexpr int kSmallMax = kSmallBlock * kSmallRounds;
+
+template <typename K, typename V, bool HAS_V>
+__global__ __launch_bounds__(kSmallBlock) void small_sort_kernel(const K *__restrict__ kin,
+                                                                 K *__restrict__ kout,
+                                                                 const V *__restrict__ vin,
+                                                                 V *__restrict__ vout, int num,
+                                                                 int begin_bit, int end_bit) {
+  constexpr int kSlots = kSmallRounds * (kSmallBlock / kWave);  // 64 (round, wave) slots
+  __shared__ K kbuf[kSmallMax];
+  __shared__ uint16_t pbuf[kSmallMax];
+  __shared__ uint32_t cnt[16 * kSlots];  // digit-major
+  __shared__ uint32_t wsum[kSmallBlock / kWave];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  K key[kSmallRounds];
+  uint32_t perm[kSmallRounds];
+#pragma unroll
+  for (int r = 0; r < kSmallRounds; ++r) {
+    const int e = r * kSmallBlock + tid;
+    key[r] = e < num ? kin[e] : (K)0;
+    perm[r] = (uint32_t)e;
+  }
+  for (int shift = begin_bit; shift < end_bit; shift += 4) {
+    const uint32_t dmask = end_bit - shift >= 4 ? 15u : ((1u << (end_bit - shift)) - 1u);
+    cnt[tid] = 0;
+    __syncthreads();
+    int rank[kSmallRounds];
+    uint32_t dig[kSmallRounds];
+#pragma unroll
+    for (int r = 0; r < kSmallRounds; ++r) {
+      const bool valid = r * kSmallBlock + tid < num;
+      const uint32_t d = (uint32_t)(key[r] >> shift) & dmask;
+      uint64_t peers = wave_ballot(valid);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const bool bit = (d >> b) & 1u;
+        const uint64_t bal = wave_ballot(bit);
+        peers &= bit ? bal : ~bal;
+      }
+      rank[r] = __popcll(peers & lt_mask);
+      dig[r] = d;
+      if (valid && rank[r] == 0) cnt[d * kSlots + r * (kSmallBlock / kWave) + wave] = (uint32_t)__popcll(peers);
+    }
+    __syncthreads();
+    // exclusive scan of the 1024 counters, one per thread
+    const int c = (int)cnt[tid];
+    const int inc = wave_inclusive_sum(c);
+    if (lane == 63) wsum[wave] = (uint32_t)inc;
+    __syncthreads();
+    uint32_t before = 0;
+    for (int w = 0; w < wave; ++w) before += wsum[w];
+    cnt[tid] = before + (uint32_t)(inc - c);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSmallRounds; ++r) {
+      if (r * kSmallBlock + tid < num) {
+        const uint32_t pos = cnt[dig[r] * kSlots + r * (kSmallBlock / kWave) + wave] + (uint32_t)rank[r];
+        kbuf[pos] = key[r];
+        pbuf[pos] = (uint16_t)perm[r];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSmallRounds; ++r) {
+      const int e = r * kSmallBlock + tid;
+      if (e < num) {
+        key[r] = kbuf[e];
+        perm[r] = pbuf[e];
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < kSmallRounds; ++r) {
+    const int e = r * kSmallBlock + tid;
+    if (e < num) {
+      kout[e] = key[r];
+      if (HAS_V) vout[e] = vin[perm[r]];
+    }
+  }
+}
+
 template <typename T>
 __global__ void copy_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t num) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -146,6 +238,16 @@ int sort_pairs(const K *kin, K *kout, const V *vin, V *vout, K *ktmp, V *vtmp, i
   const Plan p = plan(num);
   const int passes = end_bit > begin_bit ? (end_bit - begin_bit + 7) / 8 : 0;
   const bool has_v = vin != nullptr;
+  if (num <= kSmallMax) {
+    if (has_v)
+      small_sort_kernel<K, V, true><<<dim3(1), dim3(kSmallBlock), 0, st>>>(
+          kin, kout, vin, vout, (int)num, begin_bit, end_bit);
+    else
+      small_sort_kernel<K, V, false><<<dim3(1), dim3(kSmallBlock), 0, st>>>(
+          kin, kout, vin, vout, (int)num, begin_bit, end_bit);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
   if (passes == 0) {
     const unsigned g = (unsigned)ceil_div64(num, 256);
     copy_kernel<K><<<dim3(g), dim3(256), 0, st>>>(kin, kout, num);
@@ -158,17 +260,18 @@ int sort_pairs(const K *kin, K *kout, const V *vin, V *vout, K *ktmp, V *vtmp, i
   bool to_out = (passes & 1) != 0;  // alternate so that the last pass writes kout/vout
   for (int pass = 0; pass < passes; ++pass) {
     const int shift = begin_bit + 8 * pass;
+    const uint32_t dmask = end_bit - shift >= 8 ? 255u : ((1u << (end_bit - shift)) - 1u);
     K *kdst = to_out ? kout : ktmp;
     V *vdst = to_out ? vout : vtmp;
-    hist_kernel<K><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(ksrc, num, shift, p.rounds,
-                                                                     p.ntiles, hist);
+    hist_kernel<K><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(ksrc, num, shift, dmask,
+                                                                     p.rounds, p.ntiles, hist);
     hist_scan_kernel<<<dim3(1), dim3(kScanBlock), 0, st>>>(hist, p.ntiles * kBins);
     if (has_v)
       scatter_kernel<K, V, true><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(
-          ksrc, vsrc, kdst, vdst, num, shift, p.rounds, p.ntiles, hist);
+          ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, hist);
     else
       scatter_kernel<K, V, false><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(
-          ksrc, vsrc, kdst, vdst, num, shift, p.rounds, p.ntiles, hist);
+          ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, hist);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     ksrc = kdst;
     vsrc = vdst;

@@ -164,6 +164,17 @@ def sub(idxs, tss, lens, *, pad_head, ofst, span, traj_stride, step_bytes, col_b
     return outs[0], outs[1], outs[2], span * step_bytes
 
 
+def split_step_index(flat, trajectory_length, modulo=0, idxs=None, tss=None, lens=None):
+    """flat step indices -> (trajectory, timestep, length = timestep + 1) on the device."""
+    _need(flat, torch.int64, "flat")
+    num = flat.numel()
+    outs = [t if t is not None else torch.empty(num, dtype=torch.int64, device=flat.device)
+            for t in (idxs, tss, lens)]
+    call("gear_hip_split_step_index", _ptr(flat), num, int(trajectory_length), int(modulo),
+         _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _stream())
+    return outs[0], outs[1], outs[2]
+
+
 def prefix_sum(priorities, out=None):
     """fp32[n] -> inclusive fp64 prefix[n] (gear_hip_scan_f32_f64)."""
     _need(priorities, torch.float32, "priorities")

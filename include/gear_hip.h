@@ -139,6 +139,17 @@ int gear_hip_sub(int64_t num, const int64_t *idxs, const int64_t *tss, const int
                  int64_t step_bytes, int64_t col_base, int64_t *src_offsets,
                  int64_t *dst_offsets, int64_t *copy_lens, void *stream);
 
+/* Sampled flat step index -> window arguments of gear_hip_subcopy, for tables whose priorities
+ * are kept per step (BASELINE configs 4 and 5):  f = flat[j] (mod `modulo` when modulo > 0);
+ *     idxs[j] = f / trajectory_length;  tss[j] = f % trajectory_length;  lens[j] = tss[j] + 1
+ * (lens may be NULL).  lens = ts + 1 is the offline convention "timestep == length" of
+ * gear/loader/offline_loader.py:200-201,263 applied to a step inside a trajectory: the window
+ * never reaches past the sampled step.  Stands where the loader looks timesteps up on the host
+ * (gear/loader/offline_loader.py:168-177). */
+int gear_hip_split_step_index(const int64_t *flat, int64_t num, int64_t trajectory_length,
+                              int64_t modulo, int64_t *idxs, int64_t *tss, int64_t *lens,
+                              void *stream);
+
 /* ---- weighted sampler: prefix sum + search ------------------------------------------------ */
 
 /* Inclusive prefix sum of fp32 priorities accumulated and written in fp64:
