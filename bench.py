@@ -84,15 +84,13 @@ def run_config4(args):
     dsts = [torch.empty((B, span * sb), dtype=torch.uint8, device="cuda") for sb in tab.step_bytes]
     cols = [dict(dst=dsts[c], ofst=ofst, span=span, step_bytes=tab.step_bytes[c],
                  col_base=tab.col_base(c), pad_head=True, zero_fill=True) for c in range(4)]
-    key_bits = max(int(nsteps_total - 1).bit_length(), 1)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(args.steps)]
 
     def step(i, timed_slot=None):
         ops.prefix_sum(dpri, out=prefix)
-        ops.upper_bound(prefix, u01[i], unit_uniforms=True, idx_out=flat)
-        sflat = ops.sort_i64(flat, key_bits=key_bits)
-        ops.split_step_index(sflat, T, idxs=idxs, tss=tss, lens=lens)
+        ops.sample_sorted(prefix, u01[i], unit_uniforms=True, sorted_out=flat,
+                          trajectory_length=T, idxs=idxs, tss=tss, lens=lens)
         if timed_slot is not None:
             ev[timed_slot][0].record()
         ops.subcopy_multi(table, idxs, tss, lens, tab.traj_stride, cols)
@@ -125,7 +123,7 @@ def run_config4(args):
                                "priority-sampled batch of %d windows x %d steps, 4 columns"
                                % (nsteps_total, cap, T, B, span),
                    "table_bytes": tab.nbytes, "batch_payload_bytes": payload,
-                   "step": "scan(1e6 f32->f64) + search(2048) + sort + split + gather(4 columns)"},
+                   "step": "scan(1e6 f32->f64) + [search(2048) + sort + split] + gather(4 columns)"},
         "step_GBps": alg_bytes / (ms_per_step * 1e-3) / 1e9,
         "step_frac_of_hbm_peak": alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": achieved,

@@ -16,9 +16,18 @@
 namespace gearhip {
 namespace {
 
-constexpr int kBlock = 256;
+#ifndef GEARHIP_GATHER_BLOCK
+#define GEARHIP_GATHER_BLOCK 128
+#endif
+constexpr int kBlock = GEARHIP_GATHER_BLOCK;
 
 enum GatherMode { kSubcopy = 0, kVcopy = 1, kCopy = 2 };
+
+#ifdef GEARHIP_GATHER_ADJ
+#define GEARHIP_VEC_INDEX(k0, u, tg, lane, U) ((k0) + (int64_t)(lane) * (U) + (u))
+#else
+#define GEARHIP_VEC_INDEX(k0, u, tg, lane, U) ((k0) + (int64_t)(u) * (tg) + (lane))
+#endif
 
 struct ColumnArgs {
   uint8_t *dst;
@@ -54,15 +63,16 @@ struct Slice {
   int64_t n;          // copied bytes
 };
 
-template <bool NT>
+// NT is a bit mask: 1 = non-temporal loads, 2 = non-temporal stores
+template <int NT>
 __device__ __forceinline__ u32x4 load16(const uint8_t *p) {
-  if (NT) return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a1 *>(p));
+  if (NT & 1) return __builtin_nontemporal_load(reinterpret_cast<const u32x4_a1 *>(p));
   return reinterpret_cast<const u32x4_any *>(p)->v;
 }
 
-template <bool NT>
+template <int NT>
 __device__ __forceinline__ void store16(uint8_t *p, u32x4 v) {
-  if (NT)
+  if (NT & 2)
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
   else
     *reinterpret_cast<u32x4 *>(p) = v;
@@ -70,7 +80,7 @@ __device__ __forceinline__ void store16(uint8_t *p, u32x4 v) {
 
 // Copies the part of slice `s` that belongs to group-chunk `c` (and c+cps, ... if the slice is
 // longer than the launch was sized for).
-template <int U, bool NT>
+template <int U, int NT>
 __device__ __forceinline__ void gather_chunks(const Slice &s, int64_t c, int64_t cps, int lane,
                                               int tg) {
   const uintptr_t r0 = reinterpret_cast<uintptr_t>(s.rp);
@@ -85,7 +95,7 @@ __device__ __forceinline__ void gather_chunks(const Slice &s, int64_t c, int64_t
     int kind[U];  // 0 nothing, 1 full aligned store, 2 byte path
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t k = k0 + (int64_t)u * tg + lane;
+      const int64_t k = GEARHIP_VEC_INDEX(k0, u, tg, lane, U);
       const int64_t lo = (k << 4) - head;
       const int64_t hi = lo + 16;
       kind[u] = 0;
@@ -107,13 +117,13 @@ __device__ __forceinline__ void gather_chunks(const Slice &s, int64_t c, int64_t
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t k = k0 + (int64_t)u * tg + lane;
+      const int64_t k = GEARHIP_VEC_INDEX(k0, u, tg, lane, U);
       if (kind[u] == 1) store16<NT>(ap + (k << 4), v[u]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (kind[u] == 2) {
-        const int64_t k = k0 + (int64_t)u * tg + lane;
+        const int64_t k = GEARHIP_VEC_INDEX(k0, u, tg, lane, U);
         const int64_t lo = (k << 4) - head;
         for (int j = 0; j < 16; ++j) {
           const int64_t off = lo + j;
@@ -157,7 +167,7 @@ __device__ __forceinline__ Slice resolve_window(const GatherArgs &p, const Colum
   return s;
 }
 
-template <int U, bool NT>
+template <int U, int NT>
 __device__ __forceinline__ void subcopy_body(const GatherArgs &p, const ColumnArgs &col,
                                              int64_t block) {
   const int64_t t = block * kBlock + threadIdx.x;
@@ -186,23 +196,29 @@ __device__ __forceinline__ void subcopy_body(const GatherArgs &p, const ColumnAr
   gather_chunks<U, NT>(s, c, col.cps, lane, tg);
 }
 
-template <int U, bool NT>
+template <int U, int NT>
 __global__ __launch_bounds__(kBlock) void subcopy_kernel(GatherArgs p, ColumnArgs col) {
   subcopy_body<U, NT>(p, col, blockIdx.x);
 }
 
-template <int U, bool NT>
+template <int U, int NT>
 __global__ __launch_bounds__(kBlock) void subcopy_multi_kernel(GatherArgs p, MultiArgs m) {
   // columns are laid out one after another along the grid; find this block's column
   int ci = 0;
+#ifdef GEARHIP_GATHER_XCD
+  const int64_t per = (gridDim.x + 7) / 8;
+  int64_t b = (int64_t)(blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  if (b >= gridDim.x) return;
+#else
   const int64_t b = blockIdx.x;
+#endif
 #pragma unroll 1
   for (int i = 1; i < m.ncols; ++i)
     if (b >= m.col[i].block_begin) ci = i;
   subcopy_body<U, NT>(p, m.col[ci], b - m.col[ci].block_begin);
 }
 
-template <int MODE, int U, bool NT>
+template <int MODE, int U, int NT>
 __global__ __launch_bounds__(kBlock) void slices_kernel(GatherArgs p, uint8_t *dst, int64_t cps,
                                                         int tg_shift) {
   const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -289,13 +305,16 @@ Shape plan(int64_t num, int64_t max_region, int U) {
   return s;
 }
 
+// Measured on MI355X at the 2048 x 847 KB window shape: two vectors per thread (8 KiB per
+// workgroup, many small workgroups) with non-temporal stores moves 6.1 TB/s; four or eight
+// vectors per thread, or plain stores, stay between 5.1 and 5.7 TB/s.
 int pick_unroll() {
-  static int u = env_int("GEAR_HIP_GATHER_UNROLL", 8);
-  return (u == 4 || u == 8 || u == 16) ? u : 8;
+  static int u = env_int("GEAR_HIP_GATHER_UNROLL", 2);
+  return (u == 2 || u == 4 || u == 8) ? u : 2;
 }
-bool pick_nt() {
-  static int nt = env_int("GEAR_HIP_GATHER_NT", 0);
-  return nt != 0;
+int pick_nt() {
+  static int nt = env_int("GEAR_HIP_GATHER_NT", 2);
+  return nt == 0 ? 0 : 2;
 }
 
 int fill_column(const gear_hip_column_desc &d, int64_t num, int U, ColumnArgs *out,
@@ -323,46 +342,63 @@ int fill_column(const gear_hip_column_desc &d, int64_t num, int U, ColumnArgs *o
   return 0;
 }
 
-template <int U>
-int launch_subcopy_u(const GatherArgs &p, const ColumnArgs &col, int64_t blocks, bool nt,
-                     hipStream_t st) {
-  if (nt)
-    subcopy_kernel<U, true><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, col);
-  else
-    subcopy_kernel<U, false><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, col);
+template <int U, int NT>
+int launch_subcopy_un(const GatherArgs &p, const ColumnArgs &col, int64_t blocks, hipStream_t st) {
+  subcopy_kernel<U, NT><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, col);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
 
-template <int U>
-int launch_multi_u(const GatherArgs &p, const MultiArgs &m, int64_t blocks, bool nt,
-                   hipStream_t st) {
-  if (nt)
-    subcopy_multi_kernel<U, true><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, m);
-  else
-    subcopy_multi_kernel<U, false><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, m);
+template <int U, int NT>
+int launch_multi_un(const GatherArgs &p, const MultiArgs &m, int64_t blocks, hipStream_t st) {
+  subcopy_multi_kernel<U, NT><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, m);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
+}
+
+template <int MODE, int U, int NT>
+int launch_slices_un(const GatherArgs &p, uint8_t *dst, const Shape &s, hipStream_t st) {
+  slices_kernel<MODE, U, NT><<<dim3((unsigned)s.blocks), dim3(kBlock), 0, st>>>(p, dst, s.cps,
+                                                                              s.tg_shift);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+// picks the instantiation for the (unroll, non-temporal) pair chosen at run time
+#define GEARHIP_DISPATCH_U_NT(U, NT, CALL)                          \
+  do {                                                              \
+    if ((NT) == 0) {                                                \
+      if ((U) == 8) return CALL(8, 0);                              \
+      if ((U) == 4) return CALL(4, 0);                              \
+      return CALL(2, 0);                                            \
+    }                                                               \
+    if ((U) == 8) return CALL(8, 2);                                \
+    if ((U) == 4) return CALL(4, 2);                                \
+    return CALL(2, 2);                                              \
+  } while (0)
+
+int launch_subcopy(const GatherArgs &p, const ColumnArgs &col, int64_t blocks, int U, int nt,
+                   hipStream_t st) {
+#define CALL_(UU, NN) launch_subcopy_un<UU, NN>(p, col, blocks, st)
+  GEARHIP_DISPATCH_U_NT(U, nt, CALL_);
+#undef CALL_
+}
+
+int launch_multi(const GatherArgs &p, const MultiArgs &m, int64_t blocks, int U, int nt,
+                 hipStream_t st) {
+#define CALL_(UU, NN) launch_multi_un<UU, NN>(p, m, blocks, st)
+  GEARHIP_DISPATCH_U_NT(U, nt, CALL_);
+#undef CALL_
 }
 
 template <int MODE>
 int launch_slices(const GatherArgs &p, uint8_t *dst, int64_t max_len, hipStream_t st) {
-  const int U = pick_unroll();
+  const int U = pick_unroll(), nt = pick_nt();
   const Shape s = plan(p.num, max_len, U);
   if (s.blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
-  const dim3 grid((unsigned)s.blocks), block(kBlock);
-  switch (U) {
-    case 4:
-      slices_kernel<MODE, 4, false><<<grid, block, 0, st>>>(p, dst, s.cps, s.tg_shift);
-      break;
-    case 16:
-      slices_kernel<MODE, 16, false><<<grid, block, 0, st>>>(p, dst, s.cps, s.tg_shift);
-      break;
-    default:
-      slices_kernel<MODE, 8, false><<<grid, block, 0, st>>>(p, dst, s.cps, s.tg_shift);
-  }
-  GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  return 0;
+#define CALL_(UU, NN) launch_slices_un<MODE, UU, NN>(p, dst, s, st)
+  GEARHIP_DISPATCH_U_NT(U, nt, CALL_);
+#undef CALL_
 }
 
 }  // namespace
@@ -395,12 +431,7 @@ extern "C" int gear_hip_subcopy(const void *src, void *dst, int64_t num, const i
   if (rc) return rc;
   if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
   GatherArgs p{static_cast<const uint8_t *>(src), num, idxs, tss, lens, traj_stride, 0};
-  const bool nt = pick_nt();
-  switch (U) {
-    case 4: return launch_subcopy_u<4>(p, col, blocks, nt, as_stream(stream));
-    case 16: return launch_subcopy_u<16>(p, col, blocks, nt, as_stream(stream));
-    default: return launch_subcopy_u<8>(p, col, blocks, nt, as_stream(stream));
-  }
+  return launch_subcopy(p, col, blocks, U, pick_nt(), as_stream(stream));
 }
 
 extern "C" int gear_hip_subcopy_multi(const void *src, int64_t num, const int64_t *idxs,
@@ -424,12 +455,7 @@ extern "C" int gear_hip_subcopy_multi(const void *src, int64_t num, const int64_
   for (int i = ncols; i < GEAR_HIP_MAX_COLUMNS; ++i) m.col[i] = m.col[0];
   if (total >= 0x7fffffffll) return GEAR_HIP_ERANGE;
   GatherArgs p{static_cast<const uint8_t *>(src), num, idxs, tss, lens, traj_stride, 0};
-  const bool nt = pick_nt();
-  switch (U) {
-    case 4: return launch_multi_u<4>(p, m, total, nt, as_stream(stream));
-    case 16: return launch_multi_u<16>(p, m, total, nt, as_stream(stream));
-    default: return launch_multi_u<8>(p, m, total, nt, as_stream(stream));
-  }
+  return launch_multi(p, m, total, U, pick_nt(), as_stream(stream));
 }
 
 extern "C" int gear_hip_vcopy(const void *src, void *dst, int64_t num,

@@ -132,13 +132,90 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(const K *__restrict__ k
 }
 
 // ---- one-workgroup sort for small batches (a sampled batch of indices) --------------------------
-// Up to kSmallMax keys stay in registers (4 per thread, element e = r*1024 + tid) and move
-// through LDS once per 4-bit digit: ballots rank equal digits inside a wave, a 16 x 64 table of
-// (digit, round*16+wave) counts is scanned by the 1024 threads, one counter each.  The payload is
-// carried as the element's original position and applied with one global gather at the end.
+// Up to kSmallMax keys stay in registers (element e = r*1024 + tid, r < 4) and move through LDS
+// once per digit.  Ballots rank equal digits inside a wave; a digit-major table of
+// (digit, round*16+wave) counts, one counter per thread, is scanned by the workgroup.  The table
+// has 1024 counters, so the digit is 6 bits wide for up to 1024 keys, 5 bits up to 2048 and
+// 4 bits up to 4096.  The payload is carried as the element's original position.
 constexpr int kSmallBlock = 1024;
 constexpr int kSmallRounds = 4;
 constexpr int kSmallMax = kSmallBlock * kSmallRounds;
+constexpr int kSmallWaves = kSmallBlock / kWave;
+
+template <typename K>
+struct SmallSortSmem {
+  K kbuf[kSmallMax];
+  uint16_t pbuf[kSmallMax];
+  uint32_t cnt[kSmallBlock];
+  uint32_t wsum[kSmallWaves];
+};
+
+// Sorts bits [begin_bit, end_bit) of the keys held by the workgroup, stable; on return key[r] /
+// perm[r] of thread tid are the key and original position of sorted element r*1024 + tid.
+template <typename K>
+__device__ __forceinline__ void block_sort_small(K (&key)[kSmallRounds],
+                                                 uint32_t (&perm)[kSmallRounds], int num,
+                                                 int begin_bit, int end_bit,
+                                                 SmallSortSmem<K> &sm) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  const int nr = (num + kSmallBlock - 1) / kSmallBlock;  // active rounds, 1..4
+  const int dbits = nr <= 1 ? 6 : (nr == 2 ? 5 : 4);
+  const int slots = nr * kSmallWaves;
+  sm.cnt[tid] = 0;
+  __syncthreads();
+  for (int shift = begin_bit; shift < end_bit; shift += dbits) {
+    const int width = end_bit - shift >= dbits ? dbits : end_bit - shift;
+    const uint32_t dmask = (1u << width) - 1u;
+    int rank[kSmallRounds];
+    uint32_t slot[kSmallRounds];
+#pragma unroll
+    for (int r = 0; r < kSmallRounds; ++r) {
+      if (r < nr) {
+        const bool valid = r * kSmallBlock + tid < num;
+        const uint32_t d = (uint32_t)(key[r] >> shift) & dmask;
+        uint64_t peers = wave_ballot(valid);
+        for (int b = 0; b < width; ++b) {
+          const bool bit = (d >> b) & 1u;
+          const uint64_t bal = wave_ballot(bit);
+          peers &= bit ? bal : ~bal;
+        }
+        rank[r] = __popcll(peers & lt_mask);
+        slot[r] = d * slots + r * kSmallWaves + wave;
+        if (valid && rank[r] == 0) sm.cnt[slot[r]] = (uint32_t)__popcll(peers);
+      }
+    }
+    __syncthreads();
+    // exclusive scan of the counters, one per thread
+    const int c = (int)sm.cnt[tid];
+    const int inc = wave_inclusive_sum(c);
+    if (lane == 63) sm.wsum[wave] = (uint32_t)inc;
+    __syncthreads();
+    uint32_t before = 0;
+    for (int w = 0; w < wave; ++w) before += sm.wsum[w];
+    sm.cnt[tid] = before + (uint32_t)(inc - c);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSmallRounds; ++r) {
+      if (r < nr && r * kSmallBlock + tid < num) {
+        const uint32_t pos = sm.cnt[slot[r]] + (uint32_t)rank[r];
+        sm.kbuf[pos] = key[r];
+        sm.pbuf[pos] = (uint16_t)perm[r];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < kSmallRounds; ++r) {
+      const int e = r * kSmallBlock + tid;
+      if (r < nr && e < num) {
+        key[r] = sm.kbuf[e];
+        perm[r] = sm.pbuf[e];
+      }
+    }
+    sm.cnt[tid] = 0;
+    __syncthreads();
+  }
+}
 
 template <typename K, typename V, bool HAS_V>
 __global__ __launch_bounds__(kSmallBlock) void small_sort_kernel(const K *__restrict__ kin,
@@ -146,13 +223,8 @@ __global__ __launch_bounds__(kSmallBlock) void small_sort_kernel(const K *__rest
                                                                  const V *__restrict__ vin,
                                                                  V *__restrict__ vout, int num,
                                                                  int begin_bit, int end_bit) {
-  constexpr int kSlots = kSmallRounds * (kSmallBlock / kWave);  // 64 (round, wave) slots
-  __shared__ K kbuf[kSmallMax];
-  __shared__ uint16_t pbuf[kSmallMax];
-  __shared__ uint32_t cnt[16 * kSlots];  // digit-major
-  __shared__ uint32_t wsum[kSmallBlock / kWave];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  __shared__ SmallSortSmem<K> sm;
+  const int tid = threadIdx.x;
   K key[kSmallRounds];
   uint32_t perm[kSmallRounds];
 #pragma unroll
@@ -161,56 +233,7 @@ __global__ __launch_bounds__(kSmallBlock) void small_sort_kernel(const K *__rest
     key[r] = e < num ? kin[e] : (K)0;
     perm[r] = (uint32_t)e;
   }
-  for (int shift = begin_bit; shift < end_bit; shift += 4) {
-    const uint32_t dmask = end_bit - shift >= 4 ? 15u : ((1u << (end_bit - shift)) - 1u);
-    cnt[tid] = 0;
-    __syncthreads();
-    int rank[kSmallRounds];
-    uint32_t dig[kSmallRounds];
-#pragma unroll
-    for (int r = 0; r < kSmallRounds; ++r) {
-      const bool valid = r * kSmallBlock + tid < num;
-      const uint32_t d = (uint32_t)(key[r] >> shift) & dmask;
-      uint64_t peers = wave_ballot(valid);
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const bool bit = (d >> b) & 1u;
-        const uint64_t bal = wave_ballot(bit);
-        peers &= bit ? bal : ~bal;
-      }
-      rank[r] = __popcll(peers & lt_mask);
-      dig[r] = d;
-      if (valid && rank[r] == 0) cnt[d * kSlots + r * (kSmallBlock / kWave) + wave] = (uint32_t)__popcll(peers);
-    }
-    __syncthreads();
-    // exclusive scan of the 1024 counters, one per thread
-    const int c = (int)cnt[tid];
-    const int inc = wave_inclusive_sum(c);
-    if (lane == 63) wsum[wave] = (uint32_t)inc;
-    __syncthreads();
-    uint32_t before = 0;
-    for (int w = 0; w < wave; ++w) before += wsum[w];
-    cnt[tid] = before + (uint32_t)(inc - c);
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < kSmallRounds; ++r) {
-      if (r * kSmallBlock + tid < num) {
-        const uint32_t pos = cnt[dig[r] * kSlots + r * (kSmallBlock / kWave) + wave] + (uint32_t)rank[r];
-        kbuf[pos] = key[r];
-        pbuf[pos] = (uint16_t)perm[r];
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < kSmallRounds; ++r) {
-      const int e = r * kSmallBlock + tid;
-      if (e < num) {
-        key[r] = kbuf[e];
-        perm[r] = pbuf[e];
-      }
-    }
-    __syncthreads();
-  }
+  block_sort_small<K>(key, perm, num, begin_bit, end_bit, sm);
 #pragma unroll
   for (int r = 0; r < kSmallRounds; ++r) {
     const int e = r * kSmallBlock + tid;

@@ -5,7 +5,7 @@
 // (log2(n) dependent loads), which is why all draws of a batch run concurrently.
 #include <math.h>
 
-#include "wave.hpp"
+#include "radix_sort.hpp"
 
 namespace gearhip {
 namespace {
@@ -86,6 +86,79 @@ __global__ __launch_bounds__(kBlock) void search_i64_kernel(const int64_t *__res
   idx_out[j] = i;
 }
 
+// One workgroup: search the draws, sort the found indices in LDS, split them into window
+// arguments.  One launch instead of three for a batch of up to radix::kSmallMax draws.
+__global__ __launch_bounds__(radix::kSmallBlock) void sample_small_kernel(
+    const double *__restrict__ prefix, int64_t n, const float *__restrict__ u, int num, int unit,
+    int key_bits, int64_t *__restrict__ sorted_out, int64_t T, int64_t modulo,
+    int64_t *__restrict__ idxs, int64_t *__restrict__ tss, int64_t *__restrict__ lens) {
+  __shared__ radix::SmallSortSmem<uint64_t> sm;
+  const int tid = threadIdx.x;
+  const double total = prefix[n - 1];
+  uint64_t key[radix::kSmallRounds];
+  uint32_t perm[radix::kSmallRounds];
+#pragma unroll
+  for (int r = 0; r < radix::kSmallRounds; ++r) {
+    const int e = r * radix::kSmallBlock + tid;
+    key[r] = 0;
+    perm[r] = (uint32_t)e;
+    if (e < num) {
+      const double t = unit ? (double)u[e] * total : (double)u[e];
+      int64_t i = upper_bound_dev<double>(prefix, n, t);
+      if (i > n - 1) i = n - 1;
+      key[r] = (uint64_t)i;
+    }
+  }
+  radix::block_sort_small<uint64_t>(key, perm, num, 0, key_bits, sm);
+#pragma unroll
+  for (int r = 0; r < radix::kSmallRounds; ++r) {
+    const int e = r * radix::kSmallBlock + tid;
+    if (e < num) {
+      int64_t f = (int64_t)key[r];
+      if (sorted_out) sorted_out[e] = f;
+      if (T > 0) {
+        if (modulo > 0) f %= modulo;
+        const int64_t traj = f / T;
+        const int64_t ts = f - traj * T;
+        idxs[e] = traj;
+        tss[e] = ts;
+        if (lens) lens[e] = ts + 1;
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void split_sorted_kernel(const int64_t *__restrict__ flat,
+                                                              int64_t num, int64_t T,
+                                                              int64_t modulo,
+                                                              int64_t *__restrict__ idxs,
+                                                              int64_t *__restrict__ tss,
+                                                              int64_t *__restrict__ lens) {
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j >= num) return;
+  int64_t f = flat[j];
+  if (modulo > 0) f %= modulo;
+  const int64_t traj = f / T;
+  const int64_t ts = f - traj * T;
+  idxs[j] = traj;
+  tss[j] = ts;
+  if (lens) lens[j] = ts + 1;
+}
+
+struct SampleWs {
+  size_t raw, ktmp, sorted, hist, total;
+};
+SampleWs sample_ws(int64_t num) {
+  SampleWs w;
+  const size_t m = align_up((size_t)(num > 0 ? num : 1) * 8, 256);
+  w.raw = 0;
+  w.ktmp = m;
+  w.sorted = 2 * m;
+  w.hist = 3 * m;
+  w.total = 3 * m + radix::hist_bytes(num);
+  return w;
+}
+
 size_t search_ws_bytes(int64_t num) {
   if (num <= 0) return 256;
   const int64_t blocks = ceil_div64(num, kBlock);
@@ -141,5 +214,53 @@ extern "C" int gear_hip_upper_bound_i64(const int64_t *prefix, int64_t n, const 
   search_i64_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream)>>>(
       prefix, n, u, num, unit_uniforms ? 1 : 0, idx_out);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+extern "C" size_t gear_hip_sample_workspace_bytes(int64_t num) {
+  return num <= radix::kSmallMax ? 256 : sample_ws(num).total;
+}
+
+extern "C" int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const float *u,
+                                          int64_t num, int unit_uniforms, int64_t *sorted_out,
+                                          int64_t trajectory_length, int64_t modulo,
+                                          int64_t *idxs, int64_t *tss, int64_t *lens,
+                                          void *workspace, size_t workspace_bytes, void *stream) {
+  if (n < 0 || num < 0 || trajectory_length < 0 || modulo < 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (n == 0 || !prefix || !u) return GEAR_HIP_EINVAL;
+  if (trajectory_length > 0 && (!idxs || !tss)) return GEAR_HIP_EINVAL;
+  if (trajectory_length == 0 && !sorted_out) return GEAR_HIP_EINVAL;
+  int key_bits = 0;
+  while (key_bits < 63 && ((uint64_t)(n - 1) >> key_bits) != 0) ++key_bits;
+  hipStream_t st = as_stream(stream);
+  if (num <= radix::kSmallMax) {
+    sample_small_kernel<<<dim3(1), dim3(radix::kSmallBlock), 0, st>>>(
+        prefix, n, u, (int)num, unit_uniforms ? 1 : 0, key_bits, sorted_out, trajectory_length,
+        modulo, idxs, tss, lens);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  const SampleWs w = sample_ws(num);
+  if (!workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 7))
+    return GEAR_HIP_EWORKSPACE;
+  char *ws = static_cast<char *>(workspace);
+  int64_t *raw = reinterpret_cast<int64_t *>(ws + w.raw);
+  int64_t *sorted = sorted_out ? sorted_out : reinterpret_cast<int64_t *>(ws + w.sorted);
+  const int64_t blocks = ceil_div64(num, kBlock);
+  if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  search_f64_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(
+      prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  int rc = radix::sort_pairs<uint64_t, uint64_t>(
+      reinterpret_cast<const uint64_t *>(raw), reinterpret_cast<uint64_t *>(sorted), nullptr,
+      nullptr, reinterpret_cast<uint64_t *>(ws + w.ktmp), nullptr, num, 0, key_bits,
+      reinterpret_cast<uint32_t *>(ws + w.hist), st);
+  if (rc) return rc;
+  if (trajectory_length > 0) {
+    split_sorted_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(
+        sorted, num, trajectory_length, modulo, idxs, tss, lens);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  }
   return 0;
 }

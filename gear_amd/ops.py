@@ -244,6 +244,29 @@ def upper_bound(prefix, u, *, unit_uniforms=False, idx_out=None, priorities=None
     return idx_out
 
 
+def sample_sorted(prefix, u, *, unit_uniforms=True, sorted_out=None, trajectory_length=0,
+                  modulo=0, idxs=None, tss=None, lens=None):
+    """Search + ascending sort (+ split into window arguments) of one batch of draws."""
+    _need(prefix, torch.float64, "prefix")
+    _need(u, torch.float32, "u")
+    num = u.numel()
+    dev = u.device
+    if sorted_out is None:
+        sorted_out = torch.empty(num, dtype=torch.int64, device=dev)
+    if trajectory_length > 0:
+        idxs = idxs if idxs is not None else torch.empty(num, dtype=torch.int64, device=dev)
+        tss = tss if tss is not None else torch.empty(num, dtype=torch.int64, device=dev)
+        lens = lens if lens is not None else torch.empty(num, dtype=torch.int64, device=dev)
+    nbytes = load().gear_hip_sample_workspace_bytes(num)
+    ws = _ws.get("sample", nbytes, dev)
+    call("gear_hip_sample_sorted_f64", _ptr(prefix), prefix.numel(), _ptr(u), num,
+         int(bool(unit_uniforms)), _ptr(sorted_out), int(trajectory_length), int(modulo),
+         _ptr(idxs), _ptr(tss), _ptr(lens), _ptr(ws), ws.numel(), _stream())
+    if trajectory_length > 0:
+        return sorted_out, idxs, tss, lens
+    return sorted_out
+
+
 def upper_bound_i64(prefix, u, *, unit_uniforms=True, idx_out=None):
     _need(prefix, torch.int64, "prefix")
     _need(u, torch.float64 if unit_uniforms else torch.int64, "u")

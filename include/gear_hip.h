@@ -196,6 +196,19 @@ int gear_hip_upper_bound_f64(const double *prefix, int64_t n, const float *u, in
                              double beta, float *weights_out, void *workspace,
                              size_t workspace_bytes, void *stream);
 
+/* The sampler of one batch in one call: draws searched in the fp64 prefix (as
+ * gear_hip_upper_bound_f64), the found indices sorted ascending -- what every sampler of the
+ * reference returns, torch.sort(...).values, gear/sampler/global_sampler.py:131,172,195-199 --
+ * and, when trajectory_length > 0, split like gear_hip_split_step_index into idxs/tss/lens
+ * (lens may be NULL).  sorted_out may be NULL when trajectory_length > 0.
+ * Up to 4096 draws run as ONE workgroup-level kernel (search, LDS radix sort, split); larger
+ * batches use the separate kernels and need gear_hip_sample_workspace_bytes(num) of workspace. */
+size_t gear_hip_sample_workspace_bytes(int64_t num);
+int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const float *u, int64_t num,
+                               int unit_uniforms, int64_t *sorted_out, int64_t trajectory_length,
+                               int64_t modulo, int64_t *idxs, int64_t *tss, int64_t *lens,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
 /* Same search in an int64 prefix array (exact): t_j = floor(u[j] * prefix[n-1]) with u fp64 in
  * [0,1) when unit_uniforms != 0, else t_j = (int64) u[j] taken from an int64 array passed
  * through `u` (cast).  idx_out[j] = min(#{i : prefix[i] <= t_j}, n-1). */

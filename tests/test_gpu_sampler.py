@@ -196,3 +196,27 @@ def test_config3_length_weighted_trajectory_sampling(oracle):
     t2 = rng.integers(0, pre[-1], size=1024).astype(np.int64)
     idx2 = ops.upper_bound_i64(prefix, _dev(t2), unit_uniforms=False).cpu().numpy()
     assert np.array_equal(idx2, np.searchsorted(pre, t2, "right"))
+
+
+@pytest.mark.parametrize("num", [1, 100, 1024, 1025, 2048, 3000, 4096, 4097, 10_000])
+def test_sample_sorted_equals_search_then_sort(oracle, num):
+    """The one-call sampler (search + sort + split) returns exactly sort(upper_bound(draws)) and
+    the divmod split of it; 4096 and 4097 draws straddle the one-workgroup / multi-kernel paths."""
+    from gear_amd import ops
+    n, T = 777_777, 1000
+    p = _priorities(n, 77)
+    u01 = np.random.default_rng(num).random(num, dtype=np.float32)
+    announce("sample_sorted num=%d" % num)
+    prefix = ops.prefix_sum(_dev(p))
+    srt, idxs, tss, lens = ops.sample_sorted(prefix, _dev(u01), unit_uniforms=True,
+                                             trajectory_length=T, modulo=500_000)
+    plain = ops.sample_sorted(prefix, _dev(u01), unit_uniforms=True)
+    torch.cuda.synchronize()
+    pre = prefix.cpu().numpy()
+    exp = np.sort(oracle.upper_bound_f64(pre, u01, unit_uniforms=True))
+    assert np.array_equal(srt.cpu().numpy(), exp)
+    assert np.array_equal(plain.cpu().numpy(), exp)
+    f = exp % 500_000
+    assert np.array_equal(idxs.cpu().numpy(), f // T)
+    assert np.array_equal(tss.cpu().numpy(), f % T)
+    assert np.array_equal(lens.cpu().numpy(), f % T + 1)
