@@ -11,6 +11,7 @@ namespace gearhip {
 namespace {
 
 constexpr int kBlock = 256;
+constexpr int kSearchBlock = 64;  // one wave per workgroup: spreads the divergent probes over many CUs
 
 template <typename T>
 __device__ __forceinline__ int64_t upper_bound_dev(const T *__restrict__ p, int64_t n, T t) {
@@ -25,12 +26,11 @@ __device__ __forceinline__ int64_t upper_bound_dev(const T *__restrict__ p, int6
   return lo;
 }
 
-__global__ __launch_bounds__(kBlock) void search_f64_kernel(
+__global__ __launch_bounds__(kSearchBlock) void search_f64_kernel(
     const double *__restrict__ prefix, int64_t n, const float *__restrict__ u, int64_t num,
     int unit, int64_t *__restrict__ idx_out, const float *__restrict__ priorities, double beta,
     double *__restrict__ wraw, double *__restrict__ block_max) {
-  __shared__ double wmax[kBlock / kWave];
-  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t j = (int64_t)blockIdx.x * kSearchBlock + threadIdx.x;
   const double total = prefix[n - 1];
   double w = 0.0;
   if (j < num) {
@@ -44,13 +44,10 @@ __global__ __launch_bounds__(kBlock) void search_f64_kernel(
     }
   }
   if (priorities != nullptr) {
-    // block maximum of the raw weights (weights are positive, padding lanes hold 0)
+    // workgroup (= wave) maximum of the raw weights (weights are positive, padding lanes hold 0)
     double m = w;
     for (int off = 32; off > 0; off >>= 1) m = fmax(m, __shfl_xor(m, off, kWave));
-    if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = m;
-    __syncthreads();
-    if (threadIdx.x == 0)
-      block_max[blockIdx.x] = fmax(fmax(wmax[0], wmax[1]), fmax(wmax[2], wmax[3]));
+    if (threadIdx.x == 0) block_max[blockIdx.x] = m;
   }
 }
 
@@ -86,28 +83,22 @@ __global__ __launch_bounds__(kBlock) void search_i64_kernel(const int64_t *__res
   idx_out[j] = i;
 }
 
-// One workgroup: search the draws, sort the found indices in LDS, split them into window
-// arguments.  One launch instead of three for a batch of up to radix::kSmallMax draws.
-__global__ __launch_bounds__(radix::kSmallBlock) void sample_small_kernel(
-    const double *__restrict__ prefix, int64_t n, const float *__restrict__ u, int num, int unit,
-    int key_bits, int64_t *__restrict__ sorted_out, int64_t T, int64_t modulo,
-    int64_t *__restrict__ idxs, int64_t *__restrict__ tss, int64_t *__restrict__ lens) {
+// One workgroup: sort the found indices in LDS and split them into window arguments.  (The
+// search itself stays a many-workgroup kernel: its probes are divergent loads, and one CU issues
+// only about one cache line per clock.)
+__global__ __launch_bounds__(radix::kSmallBlock) void sort_split_small_kernel(
+    const int64_t *__restrict__ raw, int num, int key_bits, int64_t *__restrict__ sorted_out,
+    int64_t T, int64_t modulo, int64_t *__restrict__ idxs, int64_t *__restrict__ tss,
+    int64_t *__restrict__ lens) {
   __shared__ radix::SmallSortSmem<uint64_t> sm;
   const int tid = threadIdx.x;
-  const double total = prefix[n - 1];
   uint64_t key[radix::kSmallRounds];
   uint32_t perm[radix::kSmallRounds];
 #pragma unroll
   for (int r = 0; r < radix::kSmallRounds; ++r) {
     const int e = r * radix::kSmallBlock + tid;
-    key[r] = 0;
+    key[r] = e < num ? (uint64_t)raw[e] : 0ull;
     perm[r] = (uint32_t)e;
-    if (e < num) {
-      const double t = unit ? (double)u[e] * total : (double)u[e];
-      int64_t i = upper_bound_dev<double>(prefix, n, t);
-      if (i > n - 1) i = n - 1;
-      key[r] = (uint64_t)i;
-    }
   }
   radix::block_sort_small<uint64_t>(key, perm, num, 0, key_bits, sm);
 #pragma unroll
@@ -161,7 +152,7 @@ SampleWs sample_ws(int64_t num) {
 
 size_t search_ws_bytes(int64_t num) {
   if (num <= 0) return 256;
-  const int64_t blocks = ceil_div64(num, kBlock);
+  const int64_t blocks = ceil_div64(num, kSearchBlock);
   return align_up((size_t)num * 8, 256) + align_up((size_t)blocks * 8, 256);
 }
 
@@ -180,7 +171,8 @@ extern "C" int gear_hip_upper_bound_f64(const double *prefix, int64_t n, const f
   if (num == 0) return 0;
   if (n == 0 || !prefix || !u || !idx_out) return GEAR_HIP_EINVAL;
   if ((priorities == nullptr) != (weights_out == nullptr)) return GEAR_HIP_EINVAL;
-  const int64_t blocks = ceil_div64(num, kBlock);
+  const int64_t blocks = ceil_div64(num, kSearchBlock);
+  const int64_t nblocks = ceil_div64(num, kBlock);
   if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
   double *wraw = nullptr, *bmax = nullptr;
   if (priorities) {
@@ -192,12 +184,12 @@ extern "C" int gear_hip_upper_bound_f64(const double *prefix, int64_t n, const f
                                       align_up((size_t)num * 8, 256));
   }
   hipStream_t st = as_stream(stream);
-  search_f64_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(
+  search_f64_kernel<<<dim3((unsigned)blocks), dim3(kSearchBlock), 0, st>>>(
       prefix, n, u, num, unit_uniforms ? 1 : 0, idx_out, priorities, beta, wraw, bmax);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   if (priorities) {
-    normalise_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(wraw, bmax, (int)blocks, num,
-                                                                     weights_out);
+    normalise_kernel<<<dim3((unsigned)nblocks), dim3(kBlock), 0, st>>>(wraw, bmax, (int)blocks,
+                                                                      num, weights_out);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
   }
   return 0;
@@ -217,9 +209,7 @@ extern "C" int gear_hip_upper_bound_i64(const int64_t *prefix, int64_t n, const 
   return 0;
 }
 
-extern "C" size_t gear_hip_sample_workspace_bytes(int64_t num) {
-  return num <= radix::kSmallMax ? 256 : sample_ws(num).total;
-}
+extern "C" size_t gear_hip_sample_workspace_bytes(int64_t num) { return sample_ws(num).total; }
 
 extern "C" int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const float *u,
                                           int64_t num, int unit_uniforms, int64_t *sorted_out,
@@ -234,24 +224,24 @@ extern "C" int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const
   int key_bits = 0;
   while (key_bits < 63 && ((uint64_t)(n - 1) >> key_bits) != 0) ++key_bits;
   hipStream_t st = as_stream(stream);
-  if (num <= radix::kSmallMax) {
-    sample_small_kernel<<<dim3(1), dim3(radix::kSmallBlock), 0, st>>>(
-        prefix, n, u, (int)num, unit_uniforms ? 1 : 0, key_bits, sorted_out, trajectory_length,
-        modulo, idxs, tss, lens);
-    GEARHIP_RETURN_IF_LAUNCH_FAILED();
-    return 0;
-  }
   const SampleWs w = sample_ws(num);
   if (!workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 7))
     return GEAR_HIP_EWORKSPACE;
   char *ws = static_cast<char *>(workspace);
   int64_t *raw = reinterpret_cast<int64_t *>(ws + w.raw);
-  int64_t *sorted = sorted_out ? sorted_out : reinterpret_cast<int64_t *>(ws + w.sorted);
   const int64_t blocks = ceil_div64(num, kBlock);
-  if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
-  search_f64_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(
+  const int64_t sblocks = ceil_div64(num, kSearchBlock);
+  if (sblocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  search_f64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(
       prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  if (num <= radix::kSmallMax) {
+    sort_split_small_kernel<<<dim3(1), dim3(radix::kSmallBlock), 0, st>>>(
+        raw, (int)num, key_bits, sorted_out, trajectory_length, modulo, idxs, tss, lens);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  int64_t *sorted = sorted_out ? sorted_out : reinterpret_cast<int64_t *>(ws + w.sorted);
   int rc = radix::sort_pairs<uint64_t, uint64_t>(
       reinterpret_cast<const uint64_t *>(raw), reinterpret_cast<uint64_t *>(sorted), nullptr,
       nullptr, reinterpret_cast<uint64_t *>(ws + w.ktmp), nullptr, num, 0, key_bits,

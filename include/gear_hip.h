@@ -201,8 +201,9 @@ int gear_hip_upper_bound_f64(const double *prefix, int64_t n, const float *u, in
  * reference returns, torch.sort(...).values, gear/sampler/global_sampler.py:131,172,195-199 --
  * and, when trajectory_length > 0, split like gear_hip_split_step_index into idxs/tss/lens
  * (lens may be NULL).  sorted_out may be NULL when trajectory_length > 0.
- * Up to 4096 draws run as ONE workgroup-level kernel (search, LDS radix sort, split); larger
- * batches use the separate kernels and need gear_hip_sample_workspace_bytes(num) of workspace. */
+ * Up to 4096 draws take two launches (search over many workgroups, then one workgroup that
+ * sorts in LDS and splits); larger batches use the multi-pass radix sort.
+ * workspace: gear_hip_sample_workspace_bytes(num) bytes on the device. */
 size_t gear_hip_sample_workspace_bytes(int64_t num);
 int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const float *u, int64_t num,
                                int unit_uniforms, int64_t *sorted_out, int64_t trajectory_length,
