@@ -20,6 +20,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per gather launch on config 4, from the two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE, each scaled by a 1 GiB plain copy in the same run) summarised in
+# profiles/subcopy_multi_kernel_config4_hbm_traffic.txt
+MEASURED_GATHER_TRAFFIC_BYTES = 3536154859
 
 
 def log(msg):
@@ -97,6 +101,17 @@ def run_config4(args):
         if timed_slot is not None:
             ev[timed_slot][1].record()
 
+    if args.calibrate_copy:
+        # a plain copy of known size through the generic slice kernel: the yardstick that the
+        # FETCH_SIZE / WRITE_SIZE counters of the gather are scaled by
+        nb = 1 << 30
+        cdst = torch.empty(nb, dtype=torch.uint8, device="cuda")
+        zero = torch.zeros(1, dtype=torch.int64, device="cuda")
+        for _ in range(3):
+            ops.copy(table, cdst, zero, zero, nb)
+        torch.cuda.synchronize()
+        del cdst
+
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -129,7 +144,8 @@ def run_config4(args):
         "roofline": {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "avg_launch_ms": gather_ms, "algorithmic_bytes": alg_bytes,
-                     "traffic": args.traffic_bytes},
+                     "traffic": args.traffic_bytes if args.traffic_bytes is not None else
+                     (MEASURED_GATHER_TRAFFIC_BYTES if cap == 1000 else None)},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst)
@@ -179,6 +195,8 @@ def main():
     ap.add_argument("--trajectories", type=int, default=1000,
                     help="config 4: trajectories of 1000 steps in the table (1000 = full size)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three 1 GiB plain copies (slices kernel) before the steps")
     ap.add_argument("--traffic-bytes", type=float, default=None,
                     help="measured HBM bytes per gather launch (from rocprofv3 --pmc runs)")
     args = ap.parse_args()
