@@ -73,7 +73,8 @@ def build_libgear_ext():
     out = libgear_ext_path()
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
            "-I", INCLUDE, "-I", host, "-I", pybind11.get_include(),
-           "-I", sysconfig.get_paths()["include"]] + srcs + ["-o", out, "-ldl", "-lpthread"]
+           "-I", sysconfig.get_paths()["include"]] + srcs + [
+               "-o", out, "-L", _PKG, "-lgearhip", "-Wl,-rpath,$ORIGIN/..", "-ldl", "-lpthread"]
     _run(cmd)
     return out
 

@@ -35,6 +35,7 @@ SIGNATURES = {
     "gear_hip_host_free": (c_int, [c_void_p]),
     "gear_hip_device_alloc": (c_int, [c_size_t, ctypes.POINTER(c_void_p)]),
     "gear_hip_device_free": (c_int, [c_void_p]),
+    "gear_hip_memcpy": (c_int, [c_void_p, c_void_p, c_size_t]),
     "gear_hip_host_register": (c_int, [c_void_p, c_size_t, ctypes.POINTER(c_void_p)]),
     "gear_hip_host_unregister": (c_int, [c_void_p]),
     "gear_hip_subcopy": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_int,
@@ -49,8 +50,10 @@ SIGNATURES = {
                              c_i64, c_i64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "gear_hip_split_step_index": (c_int, [c_void_p, c_i64, c_i64, c_i64, c_void_p, c_void_p,
                                           c_void_p, c_void_p]),
+    "gear_hip_take_i64": (c_int, [c_void_p, c_i64, c_void_p, c_i64, c_i64, c_void_p, c_void_p]),
     "gear_hip_scan_workspace_bytes": (c_size_t, [c_i64]),
     "gear_hip_scan_f32_f64": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_size_t, c_void_p]),
+    "gear_hip_scan_f32_f32": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_size_t, c_void_p]),
     "gear_hip_scan_i64": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_size_t, c_void_p]),
     "gear_hip_sum_workspace_bytes": (c_size_t, [c_i64]),
     "gear_hip_sum_f32": (c_int, [c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_size_t,

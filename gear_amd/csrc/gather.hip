@@ -284,6 +284,16 @@ __global__ __launch_bounds__(kBlock) void split_kernel(const int64_t *__restrict
   if (lens) lens[j] = ts + 1;
 }
 
+// out[j] = table[idx[j]] for 8-byte elements (timesteps / global indices of the sampled batch)
+__global__ __launch_bounds__(kBlock) void take_kernel(const int64_t *__restrict__ table, int64_t n,
+                                                      const int64_t *__restrict__ idx, int64_t num,
+                                                      int64_t add, int64_t *__restrict__ out) {
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j >= num) return;
+  const int64_t i = idx[j];
+  out[j] = (i >= 0 && i < n) ? table[i] + add : 0;
+}
+
 struct Shape {
   int tg_shift;
   int64_t cps;
@@ -505,6 +515,19 @@ extern "C" int gear_hip_split_step_index(const int64_t *flat, int64_t num, int64
   if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
   split_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream)>>>(
       flat, num, trajectory_length, modulo, idxs, tss, lens);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+extern "C" int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64_t num,
+                                 int64_t add, int64_t *out, void *stream) {
+  if (n < 0 || num < 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (!table || !idx || !out) return GEAR_HIP_EINVAL;
+  const int64_t blocks = ceil_div64(num, kBlock);
+  if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  take_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream)>>>(table, n, idx, num,
+                                                                             add, out);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

@@ -89,6 +89,13 @@ extern "C" int gear_hip_device_free(void *dev_ptr) {
   return 0;
 }
 
+extern "C" int gear_hip_memcpy(void *dst, const void *src, size_t bytes) {
+  if (bytes == 0) return 0;
+  if (dst == nullptr || src == nullptr) return GEAR_HIP_EINVAL;
+  GEARHIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyDefault));
+  return 0;
+}
+
 extern "C" int gear_hip_host_register(void *host_ptr, size_t bytes, void **dev_ptr) {
   if (host_ptr == nullptr || bytes == 0) return GEAR_HIP_EINVAL;
   if (dev_ptr) *dev_ptr = nullptr;

@@ -44,6 +44,9 @@ template <> struct OutVec2<double> {
 template <> struct OutVec2<int64_t> {
   typedef int64_t type __attribute__((ext_vector_type(2), aligned(8)));
 };
+template <> struct OutVec2<float> {
+  typedef float type __attribute__((ext_vector_type(2), aligned(4)));
+};
 
 __global__ void scan_init_kernel(uint32_t *ticket, uint64_t *desc, int64_t words) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -51,15 +54,15 @@ __global__ void scan_init_kernel(uint32_t *ticket, uint64_t *desc, int64_t words
   if (i < words) desc[i] = kEmpty;
 }
 
-template <typename In, typename Acc, int VE>
+template <typename In, typename Acc, typename Out, int VE>
 __global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
-                                                      Acc *__restrict__ out, int64_t n,
+                                                      Out *__restrict__ out, int64_t n,
                                                       uint32_t *ticket, uint64_t *aggr,
                                                       uint64_t *incl) {
   constexpr int kTileElems = kRows * kBlock * VE;
   constexpr int kWaves = kBlock / kWave;
   typedef typename InVec<In, VE>::type in_vec;
-  typedef typename OutVec2<Acc>::type out_vec2;
+  typedef typename OutVec2<Out>::type out_vec2;
   __shared__ Acc wtot[kRows][kWaves];
   __shared__ Acc s_excl;
   __shared__ uint32_t s_tile;
@@ -157,14 +160,14 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
 #pragma unroll
       for (int j = 0; j < VE; j += 2) {
         out_vec2 o;
-        o[0] = b + x[r][j];
-        o[1] = b + x[r][j + 1];
+        o[0] = (Out)(b + x[r][j]);
+        o[1] = (Out)(b + x[r][j + 1]);
         *reinterpret_cast<out_vec2 *>(out + e0 + j) = o;
       }
     } else {
 #pragma unroll
       for (int j = 0; j < VE; ++j)
-        if (e0 + j < n) out[e0 + j] = b + x[r][j];
+        if (e0 + j < n) out[e0 + j] = (Out)(b + x[r][j]);
     }
   }
 }
@@ -214,15 +217,15 @@ size_t scan_ws_bytes(int64_t n) {
   return kHeaderBytes + align_up((size_t)tiles * 16, 256);
 }
 
-template <typename In, typename Acc, int VE>
-int launch_scan(const In *in, Acc *out, int64_t n, void *ws, size_t ws_bytes, hipStream_t st) {
+template <typename In, typename Acc, typename Out, int VE>
+int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hipStream_t st) {
   if (n < 0 || n > (1ll << 40)) return n < 0 ? GEAR_HIP_EINVAL : GEAR_HIP_ERANGE;
   if (n == 0) return 0;
   if (!in || !out) return GEAR_HIP_EINVAL;
   if (!ws || ws_bytes < scan_ws_bytes(n) || (reinterpret_cast<uintptr_t>(ws) & 7))
     return GEAR_HIP_EWORKSPACE;
   if ((reinterpret_cast<uintptr_t>(in) & (sizeof(In) - 1)) ||
-      (reinterpret_cast<uintptr_t>(out) & 7))
+      (reinterpret_cast<uintptr_t>(out) & (sizeof(Out) - 1)))
     return GEAR_HIP_EALIGN;
   const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
@@ -232,8 +235,8 @@ int launch_scan(const In *in, Acc *out, int64_t n, void *ws, size_t ws_bytes, hi
   scan_init_kernel<<<dim3((unsigned)ceil_div64(words, kBlock)), dim3(kBlock), 0, st>>>(ticket, aggr,
                                                                                      words);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  scan_kernel<In, Acc, VE><<<dim3((unsigned)tiles), dim3(kBlock), 0, st>>>(in, out, n, ticket, aggr,
-                                                                         incl);
+  scan_kernel<In, Acc, Out, VE><<<dim3((unsigned)tiles), dim3(kBlock), 0, st>>>(in, out, n, ticket,
+                                                                              aggr, incl);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
@@ -247,13 +250,20 @@ extern "C" size_t gear_hip_scan_workspace_bytes(int64_t n) { return scan_ws_byte
 
 extern "C" int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspace,
                                      size_t workspace_bytes, void *stream) {
-  return launch_scan<float, double, 4>(in, out, n, workspace, workspace_bytes, as_stream(stream));
+  return launch_scan<float, double, double, 4>(in, out, n, workspace, workspace_bytes,
+                                               as_stream(stream));
 }
 
 extern "C" int gear_hip_scan_i64(const int64_t *in, int64_t *out, int64_t n, void *workspace,
                                  size_t workspace_bytes, void *stream) {
-  return launch_scan<int64_t, int64_t, 2>(in, out, n, workspace, workspace_bytes,
-                                          as_stream(stream));
+  return launch_scan<int64_t, int64_t, int64_t, 2>(in, out, n, workspace, workspace_bytes,
+                                                   as_stream(stream));
+}
+
+extern "C" int gear_hip_scan_f32_f32(const float *in, float *out, int64_t n, void *workspace,
+                                     size_t workspace_bytes, void *stream) {
+  return launch_scan<float, double, float, 4>(in, out, n, workspace, workspace_bytes,
+                                              as_stream(stream));
 }
 
 extern "C" size_t gear_hip_sum_workspace_bytes(int64_t n) {

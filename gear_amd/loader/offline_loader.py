@@ -1,0 +1,181 @@
+"""OfflineLoader with the reference's interface (gear/loader/offline_loader.py:41-304).
+
+next(loader) -> (timesteps, [one tensor [batch, pattern.length, *shape] per subscribed column])
+
+What differs from the reference, on purpose (one GPU, one data-parallel rank):
+  * the sampled batch never leaves the device: trajectory lengths are looked up with a device
+    kernel instead of `iset.timesteps[indices.cpu()]` (offline_loader.py:168-177);
+  * all subscribed columns are gathered by ONE kernel launch that also writes the padding zeros,
+    so the batch tensors are torch.empty, not torch.zeros (offline_loader.py:181-189);
+  * lengths are passed as they are (the reference takes them modulo the shard capacity,
+    offline_loader.py:196-198).
+"""
+import importlib
+import logging
+import pathlib
+from typing import Any, Dict, List, Sequence, Union
+
+import torch
+
+from .. import ops
+from ..dataset import SharedDataset
+from ..dtypes import CVT_DTYPES_GEAR_TO_TORCH
+from ..libgear import core as glibc
+from ..utils import get_local_node_hashed_int32
+from .basic_loader import BasicLoader
+
+
+def ensure_dataset(dataset):
+    if isinstance(dataset, SharedDataset):
+        return dataset
+    if isinstance(dataset, (str, pathlib.Path)):
+        return SharedDataset().load(dataset)
+    raise NotImplementedError("Conversion from %r to SharedDataset is unknown" % (dataset,))
+
+
+def _as_pattern(p):
+    if isinstance(p, glibc.SubscribePattern):
+        return p
+    pad = p.get("pad", "tail")
+    opt = glibc.SubscribePattern.PadOption.tail if pad == "tail" \
+        else glibc.SubscribePattern.PadOption.head
+    return glibc.SubscribePattern(p["offset"], p["length"], opt)
+
+
+class OfflineLoader(BasicLoader):
+    @staticmethod
+    def create(data_path, batch_size: int, mpu, sampling_method: str = "Uniform", patterns=None,
+               key: Union[int, None] = None, attach: bool = True):
+        if key is None:
+            key = get_local_node_hashed_int32()
+        dataset = SharedDataset().load(data_path, key)
+        return OfflineLoader(dataset, batch_size, mpu, sampling_method, patterns)
+
+    def __init__(self, dataset, batch_size: int, mpu, sampling_method: str = "Uniform",
+                 patterns: Sequence[Dict[str, Any]] = None, logger: logging.Logger = None,
+                 timesteps_on_device: bool = False, with_mask: bool = False) -> None:
+        super().__init__(batch_size)
+        self._dataset = ensure_dataset(dataset)
+        self._handler = self._dataset._handler
+        self._table = self._dataset._table
+        self._iset = self._dataset._iset
+        spec = self._table.get_table_spec()
+        self._sub_cols = [spec.index(p["name"]) for p in patterns]
+        if any(c < 0 for c in self._sub_cols):
+            raise ValueError("a subscribed column name is not in the table")
+        self._patterns = [_as_pattern(p) for p in patterns]
+        self._handler.set(self._sub_cols, self._patterns)
+        self._mpu = mpu
+        self._dp_rank = mpu.get_data_parallel_rank()
+        self._dp_world = mpu.get_data_parallel_world_size()
+        if self._dp_world != 1:
+            raise RuntimeError("this build loads on one data-parallel rank only")
+        self._dp_capacity = self._iset.local_capacity
+        self._batch_size = batch_size
+        self._timesteps_on_device = timesteps_on_device
+        self._with_mask = with_mask
+        self._logger = logger or logging.Logger(name="OfflineLoader", level=logging.DEBUG)
+
+        self.refresh_index()
+        sampler_cls = getattr(importlib.import_module("gear_amd.sampler"),
+                              "%sSampler" % sampling_method)
+        self._sampler = sampler_cls(self._mpu, seed=42)
+        self._indices = torch.arange(self._iset.local_capacity, dtype=torch.long,
+                                     device=self._mpu.device) + self._iset.index_offset
+        self.last_masks = None
+
+    def refresh_index(self):
+        """Upload priorities and trajectory lengths after the host side changed them."""
+        self._device_weights = self._iset.weights.to(self._mpu.device)
+        self._device_timesteps = self._iset.timesteps.to(self._mpu.device)
+
+    def update_priorities(self, indices, values, unique_indices=False):
+        """weights[indices] = values on the device copy (last write wins for duplicates)."""
+        idx = indices.to(self._mpu.device, torch.int64).contiguous()
+        if self._iset.index_offset:
+            idx = idx - self._iset.index_offset
+        ops.scatter(self._device_weights, idx,
+                    values.to(self._mpu.device, torch.float32).contiguous(),
+                    unique_indices=unique_indices)
+
+    @property
+    def table_spec(self):
+        return self._table.get_table_spec() if self._table else None
+
+    def _empty_batch(self, n):
+        out = []
+        for i, col_id in enumerate(self._sub_cols):
+            cspec = self._table.get_column_spec(col_id)
+            out.append(torch.empty((n, self._patterns[i].length) + tuple(cspec.shape),
+                                   dtype=CVT_DTYPES_GEAR_TO_TORCH[cspec.dtype],
+                                   device=self._mpu.device))
+        return out
+
+    def _gather(self, local_indices, lengths):
+        n = local_indices.numel()
+        data_batch = self._empty_batch(n)
+        masks = None
+        if self._with_mask:
+            masks = [torch.empty((n, p.length), dtype=torch.uint8, device=self._mpu.device)
+                     for p in self._patterns]
+        # offline convention: timestep == length (offline_loader.py:200-201)
+        self._handler.subcopy_multi(local_indices, lengths, lengths, self._sub_cols, data_batch,
+                                    zero_fill=True, masks=masks)
+        self.last_masks = masks
+        return data_batch
+
+    def fused_iterate(self):
+        sampled = self._sampler.sync_sample(self._indices, self._device_weights,
+                                            self._batch_size * self._dp_world)
+        local = sampled
+        if self._iset.index_offset:
+            local = sampled - self._iset.index_offset
+        lengths = ops.take_i64(self._device_timesteps, local)
+        data_batch = self._gather(local, lengths)
+        timesteps = lengths if self._timesteps_on_device else lengths.cpu()
+        return timesteps, data_batch
+
+    def low_level_controlled_iterate(self):
+        """sub() on the host, then the generic slice gather (offline_loader.py:206-278)."""
+        sampled = self._sampler.sync_sample(self._indices, self._device_weights,
+                                            self._batch_size * self._dp_world).cpu()
+        local = sampled - self._iset.index_offset
+        tss = self._iset.timesteps[local]
+        return tss, self._low_level(local, tss)
+
+    def _low_level(self, local, tss):
+        n = local.numel()
+        data_batch = []
+        src_offsets = torch.zeros(n, dtype=torch.long)
+        dst_offsets = torch.zeros(n, dtype=torch.long)
+        copied_lens = torch.zeros(n, dtype=torch.long)
+        for i, col_id in enumerate(self._sub_cols):
+            cspec = self._table.get_column_spec(col_id)
+            batch = torch.zeros((n, self._patterns[i].length) + tuple(cspec.shape),
+                                dtype=CVT_DTYPES_GEAR_TO_TORCH[cspec.dtype],
+                                device=self._mpu.device)
+            max_len = self._handler.sub(local, tss, tss, col_id, src_offsets, dst_offsets,
+                                        copied_lens)
+            src = self._table.device_address or self._table.get_address()
+            glibc.vcopy(src, batch, src_offsets.to(self._mpu.device),
+                        dst_offsets.to(self._mpu.device), copied_lens.to(self._mpu.device), max_len)
+            data_batch.append(batch)
+        return data_batch
+
+    def __next__(self):
+        return self.fused_iterate()
+
+    def __iter__(self):
+        return self
+
+    def exposed_fused_iterate(self, indices):
+        indices = indices.to(self._mpu.device, torch.int64).contiguous()
+        local = indices % self._dp_capacity
+        lengths = ops.take_i64(self._device_timesteps, local)
+        return self._gather(local, lengths)
+
+    def exposed_low_level_controlled_iterate(self, indices):
+        indices = indices.cpu().to(torch.int64)
+        local = indices % self._dp_capacity
+        tss = self._iset.timesteps[local]
+        return tss, self._low_level(local, tss)

@@ -175,6 +175,17 @@ def split_step_index(flat, trajectory_length, modulo=0, idxs=None, tss=None, len
     return outs[0], outs[1], outs[2]
 
 
+def take_i64(table, idx, add=0, out=None):
+    """out[j] = table[idx[j]] + add (int64, device)."""
+    _need(table, torch.int64, "table")
+    _need(idx, torch.int64, "idx")
+    if out is None:
+        out = torch.empty(idx.numel(), dtype=torch.int64, device=idx.device)
+    call("gear_hip_take_i64", _ptr(table), table.numel(), _ptr(idx), idx.numel(), int(add),
+         _ptr(out), _stream())
+    return out
+
+
 def prefix_sum(priorities, out=None):
     """fp32[n] -> inclusive fp64 prefix[n] (gear_hip_scan_f32_f64)."""
     _need(priorities, torch.float32, "priorities")

@@ -1,0 +1,96 @@
+"""Samplers with the reference's interface (gear/sampler/global_sampler.py:87-203):
+
+    XSampler(mpu, seed=42).sync_sample(indices, weights, batch_size) -> sorted LongTensor
+
+`indices` are the global trajectory (or step) indices of the shard, `weights` their priorities.
+The reference draws with torch.randint / torch.multinomial / torch.topk and sorts the selected
+indices with torch.sort.  Here the random numbers stay an input produced by a seeded
+torch.Generator (their stream is a property of the torch version), and everything after them --
+prefix sum, search, top-k selection, look-up of the drawn indices, sort -- runs in libgearhip.so.
+Only the single-rank path exists: with a data-parallel world of 1 the reference's
+send/recv loops are empty.
+"""
+import torch
+
+from .. import ops
+
+
+def ensure_tensor(v, device, dtype=None):
+    if not isinstance(v, torch.Tensor):
+        v = torch.as_tensor(v)
+    if dtype is not None and v.dtype != dtype:
+        v = v.to(dtype)
+    return v.to(device, non_blocking=True).contiguous()
+
+
+class UniformSampler:
+    def __init__(self, mpu, seed=42) -> None:
+        self._mpu = mpu
+        self._generator = torch.Generator(mpu.device)
+        self._generator.manual_seed(seed)
+
+    def sync_sample(self, indices, weights, batch_size):
+        if self._mpu.get_data_parallel_world_size() != 1:
+            raise RuntimeError("this build samples on one data-parallel rank only")
+        return self._dp_rank_zero_sync(indices, weights, batch_size)
+
+    def _take_sorted(self, indices, positions):
+        """sort(indices[positions]) on the device."""
+        picked = ops.take_i64(indices, positions)
+        bits = 63
+        return ops.sort_i64(picked, key_bits=bits)
+
+    def _dp_rank_zero_sync(self, indices, weights, batch_size):
+        device = self._mpu.device
+        indices = ensure_tensor(indices, device, torch.int64)
+        draws = torch.randint(low=0, high=indices.size(0), size=(batch_size,),
+                              generator=self._generator, dtype=torch.long, device=device)
+        return self._take_sorted(indices, draws)
+
+
+class WeightedSampler(UniformSampler):
+    """Priority-proportional sampling with replacement: inclusive fp64 prefix sum of the
+    priorities, then upper_bound of seeded uniforms in [0, sum).  Entries with priority 0 are
+    never drawn."""
+
+    def __init__(self, mpu, seed=42) -> None:
+        super().__init__(mpu, seed)
+        self._prefix = None
+        self.last_positions = None
+
+    def _dp_rank_zero_sync(self, indices, weights, batch_size):
+        device = self._mpu.device
+        indices = ensure_tensor(indices, device, torch.int64)
+        weights = ensure_tensor(weights, device, torch.float32)
+        if self._prefix is None or self._prefix.numel() != weights.numel():
+            self._prefix = torch.empty(weights.numel(), dtype=torch.float64, device=device)
+        ops.prefix_sum(weights, out=self._prefix)
+        u = torch.rand(batch_size, generator=self._generator, dtype=torch.float32, device=device)
+        positions = ops.sample_sorted(self._prefix, u, unit_uniforms=True)
+        self.last_positions = positions
+        return self._take_sorted(indices, positions)
+
+    def sample_with_importance(self, indices, weights, batch_size, beta=0.4):
+        """Draw a batch and its importance weights (N * P(i)) ** -beta / max over the batch.
+        Returns (indices, is_weights) in draw order (not sorted), aligned element by element."""
+        device = self._mpu.device
+        indices = ensure_tensor(indices, device, torch.int64)
+        weights = ensure_tensor(weights, device, torch.float32)
+        if self._prefix is None or self._prefix.numel() != weights.numel():
+            self._prefix = torch.empty(weights.numel(), dtype=torch.float64, device=device)
+        ops.prefix_sum(weights, out=self._prefix)
+        u = torch.rand(batch_size, generator=self._generator, dtype=torch.float32, device=device)
+        positions, is_w = ops.upper_bound(self._prefix, u, unit_uniforms=True, priorities=weights,
+                                          beta=beta)
+        return ops.take_i64(indices, positions), is_w
+
+
+class TopKSampler(UniformSampler):
+    """The batch_size largest priorities (ties: smaller index first), returned as sorted indices."""
+
+    def _dp_rank_zero_sync(self, indices, weights, batch_size):
+        device = self._mpu.device
+        indices = ensure_tensor(indices, device, torch.int64)
+        weights = ensure_tensor(weights, device, torch.float32)
+        _, positions = ops.topk(weights, batch_size, sorted_by_value=False, want_values=False)
+        return self._take_sorted(indices, positions)

@@ -61,6 +61,11 @@ int gear_hip_host_free(void *host_ptr);
 int gear_hip_device_alloc(size_t bytes, void **dev_ptr);
 int gear_hip_device_free(void *dev_ptr);
 
+/* Blocking copy of `bytes` between any two of host / pinned / device memory (direction inferred
+ * from the pointers).  A set-up call for filling and reading back device-resident tables
+ * (stands where Span::copy uses memcpy on the host-resident table, include/common/span.h:73-79). */
+int gear_hip_memcpy(void *dst, const void *src, size_t bytes);
+
 /* Pin + map an existing host range (SysV shared memory segment of a TrajectoryTable).
  * Replaces the cudaHostRegister(Mapped|Portable) of gear::memory::SharedMemory::alloc
  * (src/memory/shared_memory.cc:59-61) and the cudaHostUnregister of ::free (:70).
@@ -150,6 +155,13 @@ int gear_hip_split_step_index(const int64_t *flat, int64_t num, int64_t trajecto
                               int64_t modulo, int64_t *idxs, int64_t *tss, int64_t *lens,
                               void *stream);
 
+/* out[j] = table[idx[j]] + add for int64 tables on the device (0 where idx[j] is outside [0,n)).
+ * Replaces the host-side look-ups of the sampled batch: iset.timesteps[indices.cpu()]
+ * (gear/loader/offline_loader.py:168-177) and concat_indices[draws]
+ * (gear/sampler/global_sampler.py:131,172,196). */
+int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64_t num,
+                      int64_t add, int64_t *out, void *stream);
+
 /* ---- weighted sampler: prefix sum + search ------------------------------------------------ */
 
 /* Inclusive prefix sum of fp32 priorities accumulated and written in fp64:
@@ -162,6 +174,12 @@ int gear_hip_split_step_index(const int64_t *flat, int64_t num, int64_t trajecto
  * n may be 0 (nothing is written).  n <= 2^40. */
 size_t gear_hip_scan_workspace_bytes(int64_t n);
 int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspace,
+                          size_t workspace_bytes, void *stream);
+
+/* The same scan (fp64 accumulation) with the result rounded to fp32 on output: the signature of
+ * the reference's binding, prefix_sum(FloatTensor input, FloatTensor output)
+ * (src/cuda/one_dim_prefix_sum.cu:246-278). */
+int gear_hip_scan_f32_f32(const float *in, float *out, int64_t n, void *workspace,
                           size_t workspace_bytes, void *stream);
 
 /* Same scan over int64 weights (trajectory lengths, include/index/set.h:42), exact in int64.

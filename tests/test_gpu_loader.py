@@ -1,0 +1,232 @@
+"""GPU tests of the drop-in layer: libgear.core kernel bindings, samplers and OfflineLoader,
+through the reference's own call patterns, checked against the CPU oracle."""
+import os
+
+import numpy as np
+import pytest
+
+from conftest import announce
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def _mpu():
+    from gear_amd.mpu import ModelParallelismUnit
+    return ModelParallelismUnit(device=torch.device("cuda:0"))
+
+
+def _dataset(placement, capacity=48, T=40, seed=0):
+    """obs fp32[11], actions fp32[3], done uint8 with per-trajectory lengths in [1, T]."""
+    from gear_amd.dataset import SharedDataset
+    from gear_amd.specs import TableSpec
+    tspec = TableSpec.create(trajectory_length=T, capacity=capacity, column_specs=[
+        {"shape": [11], "dtype": torch.float32, "name": "observations"},
+        {"shape": [3], "dtype": torch.float32, "name": "actions"},
+        {"shape": [], "dtype": torch.uint8, "name": "done"}])
+    ds = SharedDataset.create(tspec, key=os.getpid() + seed, placement=placement)
+    g = torch.Generator().manual_seed(seed)
+    raw = {"observations": [], "actions": [], "done": [], "len": []}
+    for i in range(capacity):
+        n = int(torch.randint(1, T + 1, (1,), generator=g))
+        obs = torch.zeros((T, 11))
+        act = torch.zeros((T, 3))
+        done = torch.zeros(T, dtype=torch.uint8)
+        obs[:n] = torch.randn((n, 11), generator=g)
+        act[:n] = torch.randn((n, 3), generator=g)
+        done[n - 1] = 1
+        ds[i] = (float(torch.rand(1, generator=g)) + 0.01, n, [obs, act, done])
+        raw["observations"].append(obs[:n]); raw["actions"].append(act[:n])
+        raw["done"].append(done[:n]); raw["len"].append(n)
+    return ds, raw
+
+
+PATTERNS = [{"name": "observations", "offset": -40, "length": 40, "pad": "tail"},
+            {"name": "actions", "offset": -40, "length": 40, "pad": "head"},
+            {"name": "done", "offset": -5, "length": 5, "pad": "head"}]
+
+
+@pytest.mark.parametrize("placement", ["pinned", "device"])
+def test_data_integrity_invariant(placement):
+    """examples/offline/single-node/misc.py:5-31 of the reference: gather every trajectory and
+    compare with the raw data, for a host-resident (zero-copy) and an HBM-resident table."""
+    from gear_amd.loader import OfflineLoader
+    announce("loader integrity placement=%s" % placement)
+    ds, raw = _dataset(placement)
+    loader = OfflineLoader(ds, 16, _mpu(), "Uniform", PATTERNS)
+    indices = torch.arange(48, dtype=torch.long)
+    loaded = loader.exposed_fused_iterate(indices)
+    torch.cuda.synchronize()
+    for tid in range(48):
+        n = raw["len"][tid]
+        obs = loaded[0][tid].cpu()
+        assert torch.equal(obs[:n], raw["observations"][tid]) and not obs[n:].any()
+        act = loaded[1][tid].cpu()
+        assert torch.equal(act[40 - n:], raw["actions"][tid]) and not act[:40 - n].any()
+        done = loaded[2][tid].cpu()
+        k = min(n, 5)
+        assert torch.equal(done[5 - k:], raw["done"][tid][n - k:]) and not done[:5 - k].any()
+    # the host sub() + vcopy path of the reference gives the same batch
+    tss, low = loader.exposed_low_level_controlled_iterate(indices)
+    torch.cuda.synchronize()
+    assert tss.tolist() == raw["len"]
+    for a, b in zip(loaded, low):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("method", ["Uniform", "Weighted", "Topk"])
+def test_next_loader_batches(oracle, method):
+    from gear_amd.loader import OfflineLoader
+    from gear_amd import sampler as smp
+    announce("next(loader) sampling=%s" % method)
+    ds, raw = _dataset("pinned", seed=3)
+    loader = OfflineLoader(ds, 32 if method != "Topk" else 16, _mpu(),
+                           "TopK" if method == "Topk" else method, PATTERNS, with_mask=True)
+    B = loader._batch_size
+    # what the sampler will return, restated with the oracle from the same seeded draws
+    gen = torch.Generator("cuda:0").manual_seed(42)
+    w = ds.weights.numpy().copy()
+    if method == "Uniform":
+        draws = torch.randint(0, 48, (B,), generator=gen, dtype=torch.long, device="cuda:0")
+        expect = np.sort(draws.cpu().numpy())
+    elif method == "Weighted":
+        u = torch.rand(B, generator=gen, dtype=torch.float32, device="cuda:0").cpu().numpy()
+        expect = np.sort(oracle.upper_bound_f64(oracle.scan_f32_f64(w), u, unit_uniforms=True))
+    else:
+        expect = oracle.topk_f32(w, B, False)[1]
+    timesteps, batch = next(loader)
+    torch.cuda.synchronize()
+    lens = np.array(raw["len"])[expect]
+    assert timesteps.tolist() == lens.tolist()
+    for i, tid in enumerate(expect):
+        n = raw["len"][tid]
+        assert torch.equal(batch[0][i, :n].cpu(), raw["observations"][tid])
+        assert torch.equal(batch[1][i, 40 - n:].cpu(), raw["actions"][tid])
+        m = loader.last_masks[0][i].cpu()
+        assert int(m.sum()) == n and bool(m[:n].all())
+    assert batch[0].shape == (B, 40, 11) and batch[2].dtype == torch.uint8
+    assert isinstance(loader._sampler, getattr(smp, type(loader._sampler).__name__))
+
+
+def test_samplers_against_oracle(oracle):
+    from gear_amd.sampler import TopKSampler, UniformSampler, WeightedSampler
+    mpu = _mpu()
+    n, B = 200_000, 2048
+    rng = np.random.default_rng(8)
+    w = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    indices = torch.arange(n, dtype=torch.long, device="cuda:0") + 1000   # shard offset 1000
+    dw = torch.from_numpy(w)
+    announce("samplers vs oracle")
+    got = WeightedSampler(mpu, seed=42).sync_sample(indices, dw, B).cpu().numpy()
+    gen = torch.Generator("cuda:0").manual_seed(42)
+    u = torch.rand(B, generator=gen, dtype=torch.float32, device="cuda:0").cpu().numpy()
+    pos = oracle.upper_bound_f64(oracle.scan_f32_f64(w), u, unit_uniforms=True)
+    assert np.array_equal(got, np.sort(pos) + 1000)
+    got = TopKSampler(mpu).sync_sample(indices, dw, 500).cpu().numpy()
+    assert np.array_equal(got, oracle.topk_f32(w, 500, False)[1] + 1000)
+    got = UniformSampler(mpu, seed=7).sync_sample(indices, dw, B).cpu().numpy()
+    gen = torch.Generator("cuda:0").manual_seed(7)
+    draws = torch.randint(0, n, (B,), generator=gen, dtype=torch.long, device="cuda:0").cpu().numpy()
+    assert np.array_equal(got, np.sort(draws) + 1000)
+    # importance weights in draw order
+    idx, isw = WeightedSampler(mpu, seed=5).sample_with_importance(indices, dw, 512, beta=0.4)
+    gen = torch.Generator("cuda:0").manual_seed(5)
+    u = torch.rand(512, generator=gen, dtype=torch.float32, device="cuda:0").cpu().numpy()
+    prefix = oracle.scan_f32_f64(w)
+    pos = oracle.upper_bound_f64(prefix, u, unit_uniforms=True)
+    assert np.array_equal(idx.cpu().numpy(), pos + 1000)
+    exp = oracle.is_weights(w, prefix[-1], pos, 0.4)
+    assert np.all(np.abs(isw.cpu().numpy() - exp) <= np.spacing(exp))
+
+
+def test_weighted_sampler_distribution():
+    """Closed form: with priorities (1, 2, 3, 4) the draw frequencies approach 0.1 .. 0.4."""
+    from gear_amd.sampler import WeightedSampler
+    s = WeightedSampler(_mpu(), seed=123)
+    idx = torch.arange(4, dtype=torch.long, device="cuda:0")
+    w = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    counts = np.zeros(4)
+    for _ in range(20):
+        got = s.sync_sample(idx, w, 4096).cpu().numpy()
+        counts += np.bincount(got, minlength=4)
+    freq = counts / counts.sum()
+    assert np.all(np.abs(freq - np.array([0.1, 0.2, 0.3, 0.4])) < 0.01)
+
+
+def test_libgear_kernel_bindings(oracle):
+    """The reference's tests/test_copy.py and tests/test_sub.py flows through libgear.core."""
+    from gear_amd.libgear import core as glibc
+    device = torch.device("cuda:0")
+    announce("libgear.core.copy_debug (reference tests/test_copy.py)")
+    data = torch.ones((32, 100, 4, 3, 2), dtype=torch.float32, device="cpu", pin_memory=True)
+    copied = torch.zeros((10, 4, 3, 2), dtype=torch.float32, device=device)
+    src_offset = torch.zeros(1, dtype=torch.long, device=device)
+    dst_offset = torch.zeros(1, dtype=torch.long, device=device)
+    stride = copied.numel() * copied.element_size() * torch.ones(1, dtype=torch.long, device=device)
+    glibc.copy_debug(data, copied, src_offset, dst_offset, stride, int(stride[0]))
+    torch.cuda.synchronize()
+    assert torch.all(copied)
+
+    announce("handler.sub + vcopy from a device tensor (reference tests/test_sub.py)")
+    cspecs = [glibc.ColumnSpec([1, 2, 3, 4], glibc.float32, "x")]
+    tspec = glibc.TableSpec(0, 1, 100, 32, 1, cspecs)
+    table = glibc.TrajectoryTable(tspec, 7, True, "host")
+    handler = glibc.get_cpu_handler(table, 32, glibc.Range(0, 0), glibc.Range(0, 32))
+    handler.set([0], [glibc.SubscribePattern(-1, 100, glibc.SubscribePattern.PadOption.head)])
+    indices = torch.arange(10, dtype=torch.long)
+    lengths = torch.ones(10, dtype=torch.long) * 10
+    so, do, cl = (torch.zeros(10, dtype=torch.long) for _ in range(3))
+    handler.sub(indices, indices.clone(), lengths, 0, so, do, cl)
+    mock_src = torch.randn((32, 100, 1, 2, 3, 4), dtype=torch.float32, device=device)
+    dst = torch.zeros((10, 100, 1, 2, 3, 4), dtype=torch.float32, device=device)
+    glibc.vcopy(glibc.MemoryPtr(mock_src.data_ptr()), dst, so.to(device), do.to(device),
+                cl.to(device), 100 * 96)
+    torch.cuda.synchronize()
+    for i in range(10):
+        start = max(i - 1, 0)
+        assert torch.equal(dst[i, 100 - (10 - start):], mock_src[i, start:10])
+        assert not dst[i, :100 - (10 - start)].any()
+
+    announce("libgear.core.sum / prefix_sum / copy")
+    rng = np.random.default_rng(2)
+    p = (rng.lognormal(0, 1, size=100_001) ** 0.6).astype(np.float32)
+    dp = torch.from_numpy(p).to(device)
+    out = torch.zeros(1, dtype=torch.float32, device=device)
+    glibc.sum(dp, out, 1)
+    assert abs(out.item() - oracle.sum_f32(p)) <= 1e-6 * oracle.sum_f32(p)
+    pre64 = torch.empty(len(p), dtype=torch.float64, device=device)
+    pre32 = torch.empty(len(p), dtype=torch.float32, device=device)
+    glibc.prefix_sum(dp, pre64)
+    glibc.prefix_sum(dp, pre32)
+    exp = oracle.scan_f32_f64(p)
+    assert np.max(np.abs(pre64.cpu().numpy() - exp) / exp) <= 1e-12
+    assert np.array_equal(pre32.cpu().numpy(), pre64.cpu().numpy().astype(np.float32))
+    src = torch.arange(4096, dtype=torch.uint8, device=device)
+    d2 = torch.zeros(64, dtype=torch.uint8, device=device)
+    glibc.copy(glibc.MemoryPtr(src.data_ptr()), d2,
+               torch.tensor([5, 300], device=device), torch.tensor([0, 32], device=device), 32)
+    torch.cuda.synchronize()
+    assert torch.equal(d2[:32], src[5:37]) and torch.equal(d2[32:], src[300:332])
+
+    announce("subcopy on a table the GPU cannot see is refused")
+    with pytest.raises(RuntimeError, match="not visible to the GPU"):
+        z = torch.zeros(10, dtype=torch.long, device=device)
+        table.connect()
+        handler.subcopy(z, z, z, 0, dst)
+
+
+def test_update_priorities_then_topk(oracle):
+    from gear_amd.loader import OfflineLoader
+    ds, raw = _dataset("pinned", seed=5)
+    loader = OfflineLoader(ds, 8, _mpu(), "TopK", PATTERNS)
+    w = ds.weights.numpy().copy()
+    idx = torch.tensor([3, 7, 3, 40, 7])
+    val = torch.tensor([9.0, 8.0, 7.5, 6.0, 9.5])
+    announce("priority update through the loader, then a top-k batch")
+    loader.update_priorities(idx, val)
+    oracle.scatter_f32(w, idx.numpy(), val.numpy())
+    assert np.array_equal(loader._device_weights.cpu().numpy(), w)
+    timesteps, batch = next(loader)
+    expect = oracle.topk_f32(w, 8, False)[1]
+    assert set([3, 7, 40]).issubset(set(expect.tolist()))
+    assert timesteps.tolist() == [raw["len"][i] for i in expect]
