@@ -187,6 +187,294 @@ def cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst):
                          os.cpu_count() or 0)}
 
 
+class GenericTable:
+    def __init__(self, step_bytes, T, capacity):
+        self.step_bytes = list(step_bytes)
+        self.T, self.capacity = T, capacity
+        self.accu = [0]
+        for b in self.step_bytes:
+            self.accu.append(self.accu[-1] + b)
+        self.traj_stride = self.accu[-1] * T
+        self.nbytes = self.traj_stride * capacity
+
+    def col_base(self, c):
+        return self.accu[c] * self.T
+
+
+def _time_steps(torch, step, steps, warmup, events=None):
+    for i in range(warmup):
+        step(i, None)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(warmup + i, i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def _line(metric_value, unit, args, ms, workload, roofline, extra=None):
+    d = {"metric": "sampled windows/sec + gather GB/s (% of HBM peak) at batch 2048, 1 MI355X",
+         "value": metric_value, "unit": unit, "n_gpus": 1, "steps": args.steps,
+         "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+         "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+         "config": {"workload": workload}, "roofline": roofline}
+    if extra:
+        d.update(extra)
+    return d
+
+
+def run_config1(args):
+    """Uniform sampling + full-trajectory gather, 4096 x 64 table, batch 256."""
+    import numpy as np
+    import torch
+    from gear_amd import ops
+    from oracle import oracle as orc
+    tab = GenericTable([68, 24, 4, 1], 64, 4096)
+    table = fill_device_table(torch, tab.nbytes, 1001)
+    B = 256
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1001)
+    draws = torch.randint(0, 4096, (args.warmup + args.steps, B), dtype=torch.int64, device="cuda",
+                          generator=g)
+    tss = torch.zeros(B, dtype=torch.int64, device="cuda")
+    lens = torch.full((B,), 64, dtype=torch.int64, device="cuda")
+    dsts = [torch.empty((B, 64 * sb), dtype=torch.uint8, device="cuda") for sb in tab.step_bytes]
+    cols = [dict(dst=dsts[c], ofst=0, span=64, step_bytes=tab.step_bytes[c],
+                 col_base=tab.col_base(c), pad_head=False) for c in range(4)]
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+
+    def step(i, slot):
+        idx = ops.sort_i64(draws[i], key_bits=12)
+        if slot is not None:
+            ev[slot][0].record()
+        ops.subcopy_multi(table, idx, tss, lens, tab.traj_stride, cols)
+        if slot is not None:
+            ev[slot][1].record()
+
+    ms = _time_steps(torch, step, args.steps, args.warmup)
+    gms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    alg = 2 * B * tab.traj_stride
+    host = table.cpu().numpy()
+    hd = [np.zeros((B, 64 * sb), np.uint8) for sb in tab.step_bytes]
+    rng = np.random.default_rng(1)
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < 3.0:
+        idx = np.sort(rng.integers(0, 4096, size=B))
+        for c in range(4):
+            orc.subcopy(host, idx, np.zeros(B, np.int64), np.full(B, 64, np.int64), False, 0, 64,
+                        tab.traj_stride, tab.step_bytes[c], tab.col_base(c), dst=hd[c])
+        n += 1
+    cpu_ms = (time.perf_counter() - t0) * 1e3 / n
+    return _line(B / (ms * 1e-3), "trajectories/s", args, ms,
+                 "config1: 4096 x 64 table (obs f32[17], act f32[6], rew f32, done u8), uniform "
+                 "batch of 256 full trajectories, sort + 4-column gather",
+                 {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": alg / (gms * 1e-3) / 1e9,
+                  "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (gms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                  "avg_launch_ms": gms, "algorithmic_bytes": alg, "traffic": None},
+                 {"cpu_baseline": {"value": B / (cpu_ms * 1e-3), "unit": "trajectories/s", "cores": 1,
+                                   "kind": "port", "ms_per_step": cpu_ms,
+                                   "sample": "%d steps of sort + 4-column memset+memcpy gather" % n}})
+
+
+def run_config2(args):
+    """Prioritized sampling: 1e6 priorities, 4096 draws, importance weights."""
+    import numpy as np
+    import torch
+    from gear_amd import ops
+    from oracle import oracle as orc
+    n, B = 1_000_000, 4096
+    rng = np.random.default_rng(1002)
+    pri = (rng.lognormal(0.0, 1.0, size=n) ** 0.6).astype(np.float32)
+    dpri = torch.from_numpy(pri).cuda()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1002)
+    u01 = torch.rand((args.warmup + args.steps, B), dtype=torch.float32, device="cuda", generator=g)
+    prefix = torch.empty(n, dtype=torch.float64, device="cuda")
+    idx = torch.empty(B, dtype=torch.int64, device="cuda")
+    w = torch.empty(B, dtype=torch.float32, device="cuda")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+
+    def step(i, slot):
+        if slot is not None:
+            ev[slot][0].record()
+        ops.prefix_sum(dpri, out=prefix)
+        if slot is not None:
+            ev[slot][1].record()
+        ops.upper_bound(prefix, u01[i], unit_uniforms=True, idx_out=idx, priorities=dpri, beta=0.4,
+                        weights_out=w)
+
+    ms = _time_steps(torch, step, args.steps, args.warmup)
+    sms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    alg = 12 * n
+    t0 = time.perf_counter()
+    k = 0
+    while time.perf_counter() - t0 < 3.0:
+        uu = rng.random(B, dtype=np.float32)
+        pre = orc.scan_f32_f64(pri)
+        ii = orc.upper_bound_f64(pre, uu, unit_uniforms=True)
+        orc.is_weights(pri, pre[-1], ii, 0.4)
+        k += 1
+    cpu_ms = (time.perf_counter() - t0) * 1e3 / k
+    return _line(B / (ms * 1e-3), "draws/s", args, ms,
+                 "config2: 1e6 fp32 priorities -> fp64 prefix (init + scan kernels), 4096 draws, "
+                 "importance weights",
+                 {"bound": "hbm", "kernel": "scan_init_kernel + scan_kernel", "achieved": alg / (sms * 1e-3) / 1e9,
+                  "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (sms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                  "avg_launch_ms": sms, "algorithmic_bytes": alg, "traffic": None},
+                 {"cpu_baseline": {"value": B / (cpu_ms * 1e-3), "unit": "draws/s", "cores": 1,
+                                   "kind": "port", "ms_per_step": cpu_ms,
+                                   "sample": "%d steps of fp64 scan + 4096 searches + weights" % k}})
+
+
+def run_config3(args):
+    """Decision-Transformer windows: 100 000 variable-length trajectories, 1024 x 20 steps + mask."""
+    import numpy as np
+    import torch
+    from gear_amd import ops
+    tab = GenericTable([68, 24, 4, 4, 4], 1000, args.trajectories3)
+    log("building %.1f GB table in HBM" % (tab.nbytes / 1e9))
+    table = fill_device_table(torch, tab.nbytes, 1003)
+    B, span = 1024, 20
+    rng = np.random.default_rng(1003)
+    lengths = torch.from_numpy(rng.integers(200, 1001, size=tab.capacity).astype(np.int64)).cuda()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1003)
+    total = args.warmup + args.steps
+    u1 = torch.rand((total, B), dtype=torch.float64, device="cuda", generator=g)
+    u2 = torch.rand((total, B), dtype=torch.float64, device="cuda", generator=g)
+    prefix = torch.empty(tab.capacity, dtype=torch.int64, device="cuda")
+    dsts = [torch.empty((B, span * sb), dtype=torch.uint8, device="cuda") for sb in tab.step_bytes]
+    mask = torch.empty((B, span), dtype=torch.uint8, device="cuda")
+    cols = [dict(dst=dsts[c], ofst=0, span=span, step_bytes=tab.step_bytes[c],
+                 col_base=tab.col_base(c), pad_head=False, mask_out=mask if c == 0 else None)
+            for c in range(5)]
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+
+    def step(i, slot):
+        ops.prefix_sum_i64(lengths, out=prefix)
+        traj = ops.upper_bound_i64(prefix, u1[i], unit_uniforms=True)
+        traj = ops.sort_i64(traj, key_bits=17)
+        lens = ops.take_i64(lengths, traj)
+        start = (u2[i] * (lens - (span - 1)).double()).long()   # synthetic start offsets (input)
+        if slot is not None:
+            ev[slot][0].record()
+        ops.subcopy_multi(table, traj, start, lens, tab.traj_stride, cols)
+        if slot is not None:
+            ev[slot][1].record()
+
+    ms = _time_steps(torch, step, args.steps, args.warmup)
+    gms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    alg = 2 * B * span * sum(tab.step_bytes) + B * span
+    return _line(B / (ms * 1e-3), "windows/s", args, ms,
+                 "config3: %d variable-length trajectories (T=1000), length-weighted int64 sampler, "
+                 "1024 windows x 20 steps x 5 columns + uint8 mask" % tab.capacity,
+                 {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": alg / (gms * 1e-3) / 1e9,
+                  "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (gms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                  "avg_launch_ms": gms, "algorithmic_bytes": alg, "traffic": None})
+
+
+def run_config5(args):
+    """Zero-copy host-resident table + priority maintenance."""
+    import ctypes
+    import numpy as np
+    import torch
+    from gear_amd import _cabi, ops
+    lib = _cabi.load()
+    T, B, span, ofst = 1000, 2048, 30, -29
+    cap = args.trajectories5
+    tab = AtariTable(T, cap)
+    host_ptr, dev_ptr = ctypes.c_void_p(), ctypes.c_void_p()
+    while True:
+        log("pinning %.1f GB of host memory" % (tab.nbytes / 1e9))
+        rc = lib.gear_hip_host_alloc(tab.nbytes, ctypes.byref(host_ptr), ctypes.byref(dev_ptr))
+        if rc == 0:
+            break
+        cap //= 2
+        if cap < 16:
+            raise RuntimeError("cannot pin a host table")
+        tab = AtariTable(T, cap)
+    # fill the host table from a 1 GiB random device buffer (byte values do not matter)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1005)
+    piece = torch.randint(0, 256, (1 << 30,), dtype=torch.uint8, device="cuda", generator=g)
+    for o in range(0, tab.nbytes, 1 << 30):
+        nb = min(1 << 30, tab.nbytes - o)
+        _cabi.call("gear_hip_memcpy", ctypes.c_void_p(host_ptr.value + o),
+                   ctypes.c_void_p(piece.data_ptr()), nb)
+    del piece
+    src = dev_ptr.value
+    npri, k, m = 10_000_000, 65_536, 65_536
+    rng = np.random.default_rng(1005)
+    pri = torch.from_numpy((rng.lognormal(0, 1, size=npri) ** 0.6).astype(np.float32)).cuda()
+    total = args.warmup + args.steps
+    upd_idx = [torch.from_numpy(rng.permutation(npri)[:m].astype(np.int64)).cuda() for _ in range(4)]
+    upd_val = [torch.from_numpy((rng.lognormal(0, 1, size=m) ** 0.6).astype(np.float32)).cuda()
+               for _ in range(4)]
+    g.manual_seed(2005)
+    u01 = torch.rand((total, B), dtype=torch.float32, device="cuda", generator=g)
+    prefix = torch.empty(npri, dtype=torch.float64, device="cuda")
+    flat = torch.empty(B, dtype=torch.int64, device="cuda")
+    idxs, tss, lens = (torch.empty(B, dtype=torch.int64, device="cuda") for _ in range(3))
+    dsts = [torch.empty((B, span * sb), dtype=torch.uint8, device="cuda") for sb in tab.step_bytes]
+    cols = [dict(dst=dsts[c], ofst=ofst, span=span, step_bytes=tab.step_bytes[c],
+                 col_base=tab.col_base(c), pad_head=True) for c in range(4)]
+    names = ["scatter", "topk", "scan", "sample", "gather"]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)]
+          for _ in range(args.steps)]
+
+    def step(i, slot):
+        e = ev[slot] if slot is not None else None
+        if e: e[0].record()
+        ops.scatter(pri, upd_idx[i % 4], upd_val[i % 4], unique_indices=True)
+        if e: e[1].record()
+        ops.topk(pri, k, sorted_by_value=True)
+        if e: e[2].record()
+        ops.prefix_sum(pri, out=prefix)
+        if e: e[3].record()
+        ops.sample_sorted(prefix, u01[i], unit_uniforms=True, sorted_out=flat,
+                          trajectory_length=T, modulo=T * cap, idxs=idxs, tss=tss, lens=lens)
+        if e: e[4].record()
+        ops.subcopy_multi(src, idxs, tss, lens, tab.traj_stride, cols)
+        if e: e[5].record()
+
+    ms = _time_steps(torch, step, args.steps, args.warmup)
+    parts = {n: sum(ev[s][j].elapsed_time(ev[s][j + 1]) for s in range(args.steps)) / args.steps
+             for j, n in enumerate(names)}
+    payload = B * span * sum(tab.step_bytes)
+    # host-link yardstick: pinned -> device copy of the same number of bytes in the same run
+    pin = torch.empty(payload, dtype=torch.uint8, pin_memory=True)
+    dev = torch.empty(payload, dtype=torch.uint8, device="cuda")
+    for _ in range(2):
+        dev.copy_(pin, non_blocking=True)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(5):
+        dev.copy_(pin, non_blocking=True)
+    b.record()
+    torch.cuda.synchronize()
+    link_gbps = payload / (a.elapsed_time(b) / 5 * 1e-3) / 1e9
+    gather_gbps = payload / (parts["gather"] * 1e-3) / 1e9
+    lib.gear_hip_host_free(host_ptr)
+    return _line(B / (ms * 1e-3), "windows/s", args, ms,
+                 "config5: %d-step Atari-shape table in pinned host memory (%.1f GB, zero-copy), per "
+                 "step scatter 65536 -> top-65536 of 1e7 -> rescan 1e7 -> 2048 draws -> gather"
+                 % (T * cap, tab.nbytes / 1e9),
+                 {"bound": "host-link", "kernel": "subcopy_multi_kernel (source in host memory)",
+                  "achieved": gather_gbps, "peak": link_gbps, "unit": "GB/s",
+                  "frac": gather_gbps / link_gbps, "avg_launch_ms": parts["gather"],
+                  "algorithmic_bytes": payload,
+                  "peak_source": "pinned hipMemcpyAsync H2D of the same bytes in this run",
+                  "traffic": None},
+                 {"parts_ms": parts,
+                  "maintenance": {"topk_GBps_one_read": 4 * npri / (parts["topk"] * 1e-3) / 1e9,
+                                  "rescan_GBps": 12 * npri / (parts["scan"] * 1e-3) / 1e9}})
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -194,6 +482,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--trajectories", type=int, default=1000,
                     help="config 4: trajectories of 1000 steps in the table (1000 = full size)")
+    ap.add_argument("--workload", default="config4",
+                    choices=["config1", "config2", "config3", "config4", "config5"],
+                    help="BASELINE config to run (config4 is the bench line)")
+    ap.add_argument("--trajectories3", type=int, default=100_000,
+                    help="config 3: number of trajectories (100000 = full size, 10.4 GB)")
+    ap.add_argument("--trajectories5", type=int, default=2000,
+                    help="config 5: trajectories of 1000 steps in pinned host memory (2000 = 56.5 GB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB plain copies (slices kernel) before the steps")
@@ -204,7 +499,9 @@ def main():
         print("bench.py: this build runs the hot path on ONE GPU only; --gpus %d is not supported"
               % args.gpus, file=sys.stderr)
         sys.exit(2)
-    result = run_config4(args)
+    runner = {"config1": run_config1, "config2": run_config2, "config3": run_config3,
+              "config4": run_config4, "config5": run_config5}[args.workload]
+    result = runner(args)
     print(json.dumps(result), flush=True)
 
 
