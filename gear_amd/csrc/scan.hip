@@ -48,6 +48,51 @@ template <> struct OutVec2<float> {
   typedef float type __attribute__((ext_vector_type(2), aligned(4)));
 };
 
+// Writes the VE consecutive results of every lane of a wave (a contiguous slice of 64*VE
+// elements starting at e_wave) so that each store instruction covers one contiguous run:
+// non-temporal stores only reach full bandwidth when a wave writes whole cache lines.  With
+// 16 bytes per lane the lanes already do; with 32 bytes per lane (fp64 results of a float4) the
+// slice takes a detour through a wave-private LDS row.
+template <typename Out, int VE>
+__device__ __forceinline__ void store_slice(Out *__restrict__ out, int64_t e_wave, int64_t n,
+                                            const Out (&v)[VE], Out *stage_row, int lane) {
+  typedef typename OutVec2<Out>::type out_vec2;
+  constexpr int kLaneBytes = VE * (int)sizeof(Out);
+  const int64_t e0 = e_wave + (int64_t)lane * VE;
+  if (e_wave + (int64_t)kWave * VE > n) {  // ragged end of the input
+#pragma unroll
+    for (int j = 0; j < VE; ++j)
+      if (e0 + j < n) out[e0 + j] = v[j];
+    return;
+  }
+  if (kLaneBytes <= 16) {
+#pragma unroll
+    for (int j = 0; j < VE; j += 2) {
+      out_vec2 o;
+      o[0] = v[j];
+      o[1] = v[j + 1];
+      __builtin_nontemporal_store(o, reinterpret_cast<out_vec2 *>(out + e0 + j));
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VE; ++j) stage_row[lane * VE + j] = v[j];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int h = 0; h < VE / 2; ++h) {
+      out_vec2 o;
+      o[0] = stage_row[h * 2 * kWave + 2 * lane];
+      o[1] = stage_row[h * 2 * kWave + 2 * lane + 1];
+      __builtin_nontemporal_store(
+          o, reinterpret_cast<out_vec2 *>(out + e_wave + (int64_t)h * 2 * kWave + 2 * lane));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+}
+
 __global__ void scan_init_kernel(uint32_t *ticket, uint64_t *desc, int64_t words) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i == 0) *ticket = 0u;
@@ -62,8 +107,8 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
   constexpr int kTileElems = kRows * kBlock * VE;
   constexpr int kWaves = kBlock / kWave;
   typedef typename InVec<In, VE>::type in_vec;
-  typedef typename OutVec2<Out>::type out_vec2;
   __shared__ Acc wtot[kRows][kWaves];
+  __shared__ Out stage[kWaves][kWave * VE];
   __shared__ Acc s_excl;
   __shared__ uint32_t s_tile;
 
@@ -154,21 +199,113 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
 
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
     const Acc b = excl + mybase[r];
-    if (e0 + VE <= n) {
+    Out o[VE];
 #pragma unroll
-      for (int j = 0; j < VE; j += 2) {
-        out_vec2 o;
-        o[0] = (Out)(b + x[r][j]);
-        o[1] = (Out)(b + x[r][j + 1]);
-        *reinterpret_cast<out_vec2 *>(out + e0 + j) = o;
-      }
+    for (int j = 0; j < VE; ++j) o[j] = (Out)(b + x[r][j]);
+    store_slice<Out, VE>(out, base + ((int64_t)r * kBlock + wave * kWave) * VE, n, o, stage[wave],
+                         lane);
+  }
+}
+
+// ---- range variant -------------------------------------------------------------------------------
+// For up to kMaxRanges workgroups the look-back chain is not needed at all: a workgroup owns NR
+// rows of 256 vectors kept in registers, publishes the sum of its range as soon as it has loaded
+// it, and takes its exclusive prefix as the sum of ALL earlier ranges' aggregates (each thread
+// polls its share of them, fixed summation order).  Nobody waits for an inclusive value, so there
+// is no serial chain across the XCDs, and the result is bit-reproducible from run to run.
+constexpr int kMaxRanges = 2048;
+
+template <typename In, typename Acc, typename Out, int VE, int NR>
+__global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restrict__ in,
+                                                             Out *__restrict__ out, int64_t n,
+                                                             uint32_t *ticket, uint64_t *aggr) {
+  constexpr int kElems = NR * kBlock * VE;
+  constexpr int kWaves = kBlock / kWave;
+  typedef typename InVec<In, VE>::type in_vec;
+  __shared__ Acc wtot[NR][kWaves];
+  __shared__ Out stage[kWaves][kWave * VE];
+  __shared__ Acc red[kWaves];
+  __shared__ uint32_t s_tile;
+
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+  __syncthreads();
+  const int64_t tile = s_tile;
+  const int64_t base = tile * kElems;
+
+  In raw[NR][VE];
+  Acc s[NR];
+  Acc tsum = (Acc)0;
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
+    if (e0 + VE <= n) {
+      const in_vec v = __builtin_nontemporal_load(reinterpret_cast<const in_vec *>(in + e0));
+#pragma unroll
+      for (int j = 0; j < VE; ++j) raw[r][j] = v[j];
     } else {
 #pragma unroll
-      for (int j = 0; j < VE; ++j)
-        if (e0 + j < n) out[e0 + j] = (Out)(b + x[r][j]);
+      for (int j = 0; j < VE; ++j) raw[r][j] = (e0 + j < n) ? in[e0 + j] : (In)0;
     }
+  }
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    Acc a = (Acc)raw[r][0];
+#pragma unroll
+    for (int j = 1; j < VE; ++j) a += (Acc)raw[r][j];
+    s[r] = a;
+    tsum += a;
+  }
+  // the range's aggregate goes out before the detailed scan
+  {
+    const Acc w = wave_sum(tsum);
+    if (lane == 0) red[wave] = w;
+    __syncthreads();
+    if (tid == 0) store_agent(&aggr[tile], Bits<Acc>::to((red[0] + red[1]) + (red[2] + red[3])));
+  }
+  Acc wexcl[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const Acc inc = wave_inclusive_sum(s[r]);
+    wexcl[r] = wave_shift_up1(inc);
+    if (lane == kWave - 1) wtot[r][wave] = inc;
+  }
+  // sum of every earlier range (thread t takes ranges t, t+256, ...)
+  Acc part = (Acc)0;
+  for (int64_t j = tid; j < tile; j += kBlock) {
+    uint64_t v = load_agent(&aggr[j]);
+    while (v == kEmpty) {
+      __builtin_amdgcn_s_sleep(1);
+      v = load_agent(&aggr[j]);
+    }
+    part += Bits<Acc>::from(v);
+  }
+  const Acc pw = wave_sum(part);
+  __syncthreads();  // wtot complete; everybody is done reading red
+  if (lane == 0) red[wave] = pw;
+  __syncthreads();
+  const Acc excl = (red[0] + red[1]) + (red[2] + red[3]);
+
+  Acc rowbase = excl;
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    Acc acc = rowbase, mine = rowbase;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      if (w == wave) mine = acc + wexcl[r];
+      acc += wtot[r][w];
+    }
+    rowbase = acc;
+    Acc run = mine;
+    Out o[VE];
+#pragma unroll
+    for (int j = 0; j < VE; ++j) {
+      run += (Acc)raw[r][j];
+      o[j] = (Out)run;
+    }
+    store_slice<Out, VE>(out, base + ((int64_t)r * kBlock + wave * kWave) * VE, n, o, stage[wave],
+                         lane);
   }
 }
 
@@ -217,6 +354,20 @@ size_t scan_ws_bytes(int64_t n) {
   return kHeaderBytes + align_up((size_t)tiles * 16, 256);
 }
 
+template <typename In, typename Acc, typename Out, int VE, int NR>
+int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st) {
+  const int64_t ranges = ceil_div64(n, (int64_t)NR * kBlock * VE);
+  uint32_t *ticket = static_cast<uint32_t *>(ws);
+  uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
+  scan_init_kernel<<<dim3((unsigned)ceil_div64(ranges, kBlock)), dim3(kBlock), 0, st>>>(ticket, aggr,
+                                                                                      ranges);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  scan_ranges_kernel<In, Acc, Out, VE, NR><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(
+      in, out, n, ticket, aggr);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
 template <typename In, typename Acc, typename Out, int VE>
 int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hipStream_t st) {
   if (n < 0 || n > (1ll << 40)) return n < 0 ? GEAR_HIP_EINVAL : GEAR_HIP_ERANGE;
@@ -227,6 +378,16 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
   if ((reinterpret_cast<uintptr_t>(in) & (sizeof(In) - 1)) ||
       (reinterpret_cast<uintptr_t>(out) & (sizeof(Out) - 1)))
     return GEAR_HIP_EALIGN;
+  // few enough ranges: no look-back chain (4, 8 or 16 rows of 256 vectors per workgroup)
+  const int64_t row = (int64_t)kBlock * VE;
+  static const int force_nr = env_int("GEAR_HIP_SCAN_ROWS", 0);  // experiments only
+  if (force_nr == 4) return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st);
+  if (force_nr == 8) return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st);
+  if (force_nr == 16) return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st);
+  if (ceil_div64(n, 4 * row) <= 1024) return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st);
+  if (ceil_div64(n, 8 * row) <= 1024) return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st);
+  if (ceil_div64(n, 16 * row) <= kMaxRanges)
+    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st);
   const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
   uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);

@@ -16,7 +16,7 @@ constexpr int kBlock = 256;
 constexpr int kRows = 4;
 constexpr int kTile = kBlock * kRows * 4;  // elements per compaction tile
 constexpr int kHistBins = 2048;
-constexpr int kMaxHistBlocks = 1024;
+constexpr int kMaxHistBlocks = 512;
 
 struct State {
   uint32_t prefix;   // key bits decided so far (right-aligned)
@@ -61,17 +61,17 @@ __global__ void zero_kernel(uint32_t *p, int64_t words) {
 }
 
 // PASS 0: bits 31..21, PASS 1: bits 20..10 of keys whose top 11 bits equal state->prefix,
-// PASS 2: bits 9..0 of keys whose top 22 bits equal state->prefix.
+// PASS 2: bits 9..0 of keys whose top 22 bits equal state->prefix.  Workgroups count into LDS and
+// add their non-empty bins to the global histogram; the bin is picked by select_pick_kernel in a
+// launch of its own (a device-scope fence per workgroup for a "last workgroup picks" scheme costs
+// far more on this multi-XCD part than one small launch).
 template <int PASS>
 __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__restrict__ p,
-                                                             int64_t n, int64_t k, State *state,
+                                                             int64_t n, const State *state,
                                                              uint32_t *hist) {
   constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
-  constexpr int kPerThread = kBinsHere / kBlock;
   typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
   __shared__ uint32_t h[kBinsHere];
-  __shared__ uint32_t wsum[kBlock / kWave];
-  __shared__ bool s_last;
   const int tid = threadIdx.x;
   for (int i = tid; i < kBinsHere; i += kBlock) h[i] = 0;
   __syncthreads();
@@ -99,23 +99,25 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__rest
   __syncthreads();
   for (int i = tid; i < kBinsHere; i += kBlock)
     if (h[i]) atomicAdd(&hist[i], h[i]);
+}
 
-  // the last workgroup to get here picks the bin
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) s_last = atomicAdd(&state->done[PASS], 1u) == gridDim.x - 1;
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();
-
+// One workgroup: walk the histogram from the top bin down and stop at the bin that holds the
+// k_rem-th largest remaining key.
+template <int PASS>
+__global__ __launch_bounds__(kBlock) void select_pick_kernel(int64_t k, State *state,
+                                                             const uint32_t *hist) {
+  constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
+  constexpr int kPerThread = kBinsHere / kBlock;
+  __shared__ uint32_t wsum[kBlock / kWave];
+  const int tid = threadIdx.x;
+  const uint32_t prefix = PASS == 0 ? 0u : state->prefix;
   const uint32_t k_rem = PASS == 0 ? (uint32_t)k : state->k_rem;
   // thread t owns bins top-down: kBinsHere-1 - t*kPerThread - j
   uint32_t c[kPerThread];
   int tsum = 0;
 #pragma unroll
   for (int j = 0; j < kPerThread; ++j) {
-    c[j] = __hip_atomic_load(&hist[kBinsHere - 1 - tid * kPerThread - j], __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
+    c[j] = hist[kBinsHere - 1 - tid * kPerThread - j];
     tsum += (int)c[j];
   }
   const int inc = wave_inclusive_sum(tsum);
@@ -259,6 +261,121 @@ __global__ __launch_bounds__(kBlock) void compact_kernel(
   }
 }
 
+// Range variant of the compaction (cf. the range variant of the prefix sum): with at most
+// kMaxRanges workgroups every workgroup publishes its packed (greater, equal) count and takes the
+// sum of all earlier ranges' counts; no chain of inclusive values across the XCDs.
+constexpr int kMaxRanges = 2048;
+constexpr uint64_t kRangeReady = 1ull << 63;
+
+template <bool DIRECT, int NR>
+__global__ __launch_bounds__(kBlock) void compact_ranges_kernel(
+    const float *__restrict__ p, int64_t n, State *state, uint64_t *desc,
+    uint32_t *__restrict__ ckey, uint32_t *__restrict__ cidx, float *__restrict__ values_out,
+    int64_t *__restrict__ indices_out) {
+  typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
+  constexpr int kWaves = kBlock / kWave;
+  constexpr int kElems = NR * kBlock * 4;
+  __shared__ int wtot[NR][kWaves];
+  __shared__ int64_t red[kWaves];
+  __shared__ uint32_t s_tile;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) s_tile = atomicAdd(&state->ticket, 1u);
+  __syncthreads();
+  const int64_t tile = s_tile;
+  const int64_t base = tile * kElems;
+  const uint32_t thr = state->prefix;
+  const uint32_t need_eq = state->k_rem;
+
+  float q[NR][4];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * 4;
+    if (e0 + 4 <= n) {
+      const f4 v = *reinterpret_cast<const f4 *>(p + e0);
+      q[r][0] = v[0]; q[r][1] = v[1]; q[r][2] = v[2]; q[r][3] = v[3];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q[r][j] = (e0 + j < n) ? p[e0 + j] : 0.0f;
+    }
+  }
+  int s[NR];  // packed counts of the thread's vector: greater << 16 | equal
+  int64_t tsum = 0;  // greater << 31 | equal over the thread's vectors
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * 4;
+    s[r] = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t key = order_key(q[r][j]);
+      if (e0 + j < n) s[r] += key > thr ? (1 << 16) : (key == thr ? 1 : 0);
+    }
+    tsum += ((int64_t)(s[r] >> 16) << 31) | (int64_t)(s[r] & 0xffff);
+  }
+  {
+    const int64_t w = wave_sum(tsum);
+    if (lane == 0) red[wave] = w;
+    __syncthreads();
+    if (tid == 0)
+      store_agent(&desc[tile], kRangeReady | (uint64_t)(red[0] + red[1] + red[2] + red[3]));
+  }
+  int wexcl[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int inc = wave_inclusive_sum(s[r]);
+    wexcl[r] = wave_shift_up1(inc);
+    if (lane == kWave - 1) wtot[r][wave] = inc;
+  }
+  int64_t part = 0;
+  for (int64_t j = tid; j < tile; j += kBlock) {
+    uint64_t v = load_agent(&desc[j]);
+    while (!(v & kRangeReady)) {
+      __builtin_amdgcn_s_sleep(1);
+      v = load_agent(&desc[j]);
+    }
+    part += (int64_t)(v & ~kRangeReady);
+  }
+  const int64_t pw = wave_sum(part);
+  __syncthreads();
+  if (lane == 0) red[wave] = pw;
+  __syncthreads();
+  const int64_t excl = red[0] + red[1] + red[2] + red[3];
+  uint32_t gt_row = (uint32_t)(excl >> 31), eq_row = (uint32_t)(excl & 0x7fffffff);
+
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    int before = 0, mine = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      if (w == wave) mine = before + wexcl[r];
+      before += wtot[r][w];
+    }
+    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * 4;
+    uint32_t gt = gt_row + ((uint32_t)mine >> 16);
+    uint32_t eq = eq_row + ((uint32_t)mine & 0xffffu);
+    gt_row += (uint32_t)before >> 16;
+    eq_row += (uint32_t)before & 0xffffu;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (e0 + j < n) {
+        const uint32_t key = order_key(q[r][j]);
+        const bool is_gt = key > thr, is_eq = key == thr;
+        if (is_gt || (is_eq && eq < need_eq)) {
+          const uint32_t pos = gt + (eq < need_eq ? eq : need_eq);
+          if (DIRECT) {
+            indices_out[pos] = e0 + j;
+            if (values_out) values_out[pos] = q[r][j];
+          } else {
+            ckey[pos] = ~key;
+            cidx[pos] = (uint32_t)(e0 + j);
+          }
+        }
+        gt += is_gt;
+        eq += is_eq;
+      }
+    }
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void emit_kernel(const float *__restrict__ p,
                                                       const uint32_t *__restrict__ sidx, int64_t k,
                                                       float *__restrict__ values_out,
@@ -297,27 +414,53 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   const int64_t zero_words = (int64_t)(l.ckey / 4);  // header + histograms + descriptors
   zero_kernel<<<dim3((unsigned)ceil_div64(zero_words, 256)), dim3(256), 0, st>>>(
       reinterpret_cast<uint32_t *>(ws), zero_words);
-  int64_t hblocks = ceil_div64(n, (int64_t)kBlock * 4 * 8);
+  int64_t hblocks = ceil_div64(n, (int64_t)kBlock * 4 * 4);
   if (hblocks < 1) hblocks = 1;
   if (hblocks > kMaxHistBlocks) hblocks = kMaxHistBlocks;
-  const dim3 hgrid((unsigned)hblocks), block(kBlock);
-  select_hist_kernel<0><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist);
-  select_hist_kernel<1><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist + kHistBins);
-  select_hist_kernel<2><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins);
+  const dim3 hgrid((unsigned)hblocks), block(kBlock), one(1);
+  select_hist_kernel<0><<<hgrid, block, 0, st>>>(priorities, n, state, hist);
+  select_pick_kernel<0><<<one, block, 0, st>>>(k, state, hist);
+  select_hist_kernel<1><<<hgrid, block, 0, st>>>(priorities, n, state, hist + kHistBins);
+  select_pick_kernel<1><<<one, block, 0, st>>>(k, state, hist + kHistBins);
+  select_hist_kernel<2><<<hgrid, block, 0, st>>>(priorities, n, state, hist + 2 * kHistBins);
+  select_pick_kernel<2><<<one, block, 0, st>>>(k, state, hist + 2 * kHistBins);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
 
-  const int64_t tiles = ceil_div64(n, kTile);
   uint32_t *ckey = reinterpret_cast<uint32_t *>(ws + l.ckey);
   uint32_t *cidx = reinterpret_cast<uint32_t *>(ws + l.cidx);
-  if (!sorted_by_value) {
-    compact_kernel<true><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, state, desc, ckey,
-                                                                  cidx, values_out, indices_out);
-    GEARHIP_RETURN_IF_LAUNCH_FAILED();
-    return 0;
+  const bool direct = !sorted_by_value;
+  const int64_t row = (int64_t)kBlock * 4;
+#define GEARHIP_COMPACT_RANGES(NR)                                                              \
+  do {                                                                                          \
+    const unsigned g = (unsigned)ceil_div64(n, (NR) * row);                                     \
+    if (direct)                                                                                 \
+      compact_ranges_kernel<true, NR><<<dim3(g), block, 0, st>>>(priorities, n, state, desc,    \
+                                                                 ckey, cidx, values_out,        \
+                                                                 indices_out);                  \
+    else                                                                                        \
+      compact_ranges_kernel<false, NR><<<dim3(g), block, 0, st>>>(priorities, n, state, desc,   \
+                                                                  ckey, cidx, values_out,       \
+                                                                  indices_out);                 \
+  } while (0)
+  if (ceil_div64(n, 4 * row) <= 1024) {
+    GEARHIP_COMPACT_RANGES(4);
+  } else if (ceil_div64(n, 8 * row) <= 1024) {
+    GEARHIP_COMPACT_RANGES(8);
+  } else if (ceil_div64(n, 16 * row) <= kMaxRanges) {
+    GEARHIP_COMPACT_RANGES(16);
+  } else {
+    const int64_t tiles = ceil_div64(n, kTile);
+    if (direct)
+      compact_kernel<true><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, state, desc, ckey,
+                                                                    cidx, values_out, indices_out);
+    else
+      compact_kernel<false><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, state, desc,
+                                                                     ckey, cidx, values_out,
+                                                                     indices_out);
   }
-  compact_kernel<false><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, state, desc, ckey,
-                                                                 cidx, values_out, indices_out);
+#undef GEARHIP_COMPACT_RANGES
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  if (direct) return 0;
   uint32_t *skey = reinterpret_cast<uint32_t *>(ws + l.skey);
   uint32_t *sidx = reinterpret_cast<uint32_t *>(ws + l.sidx);
   int rc = radix::sort_pairs<uint32_t, uint32_t>(
