@@ -8,8 +8,10 @@
 // global_load_dwordx4 at whatever byte alignment the table layout gives (the table has no
 // padding: a window of fp32[17] steps starts on a 4-byte boundary, a uint8 column on any byte).
 // Vectors that straddle the region edge or the copy/padding edge (at most four per slice) take a
-// byte path.  A group of `tg` threads (power of two, 1..256) owns one chunk of tg*U consecutive
-// vectors; lanes of a group take consecutive vectors so a wave reads and writes 1 KiB runs.
+// byte path.  A group of `tg` threads (power of two, 1..128) owns one chunk of tg*U consecutive
+// vectors; lanes of a group take consecutive vectors so a wave reads and writes 1 KiB runs and a
+// 128-thread workgroup covers one contiguous 4 KiB piece of a large window (source cache lines
+// shared by neighbouring pieces are then fetched twice only at 4 KiB boundaries).
 // Each thread issues its U loads before its first store to keep U*16 bytes per lane in flight.
 #include "common.hpp"
 
@@ -20,6 +22,9 @@ namespace {
 #define GEARHIP_GATHER_BLOCK 128
 #endif
 constexpr int kBlock = GEARHIP_GATHER_BLOCK;
+#ifndef GEARHIP_GATHER_TG_MAX_SHIFT
+#define GEARHIP_GATHER_TG_MAX_SHIFT 7
+#endif
 
 enum GatherMode { kSubcopy = 0, kVcopy = 1, kCopy = 2 };
 
@@ -307,7 +312,7 @@ Shape plan(int64_t num, int64_t max_region, int U) {
   if (nvec < 1) nvec = 1;
   int64_t want = ceil_div64(nvec, U);
   int sh = 0;
-  while ((1ll << sh) < want && sh < 8) ++sh;
+  while ((1ll << sh) < want && sh < GEARHIP_GATHER_TG_MAX_SHIFT) ++sh;
   s.tg_shift = sh;
   s.cps = ceil_div64(nvec, (int64_t)U << sh);
   const int64_t threads = num * s.cps * (1ll << sh);
