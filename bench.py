@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per gather launch on config 4, from the two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by a 1 GiB plain copy in the same run) summarised in
 # profiles/subcopy_multi_kernel_config4_hbm_traffic.txt
-MEASURED_GATHER_TRAFFIC_BYTES = 3536154859
+MEASURED_GATHER_TRAFFIC_BYTES = 3486605072
 
 
 def log(msg):
@@ -148,12 +148,14 @@ def run_config4(args):
                 ops.subcopy_multi(table, ix, ts, ln, tab.traj_stride, cols)
                 gathered[j].record(s_gather)
 
-    run_pipelined(0, args.warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_pipelined(args.warmup, args.steps)
-    torch.cuda.synchronize()
-    ms_pipelined = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_pipelined = None
+    if not args.no_pipelined:
+        run_pipelined(0, args.warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_pipelined(args.warmup, args.steps)
+        torch.cuda.synchronize()
+        ms_pipelined = (time.perf_counter() - t0) * 1e3 / args.steps
 
     payload = B * span * sum(tab.step_bytes)
     alg_bytes = 2 * payload  # every gathered byte is read once and written once
@@ -171,9 +173,10 @@ def run_config4(args):
                                % (nsteps_total, cap, T, B, span),
                    "table_bytes": tab.nbytes, "batch_payload_bytes": payload,
                    "step": "scan(1e6 f32->f64) + [search(2048) + sort + split] + gather(4 columns)"},
-        "pipelined": {"ms_per_step": ms_pipelined, "value": B / (ms_pipelined * 1e-3),
-                      "frac_of_hbm_peak": alg_bytes / (ms_pipelined * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                      "what": "same steps, sampler of batch i+1 on a second stream during gather i"},
+        "pipelined": None if ms_pipelined is None else {
+            "ms_per_step": ms_pipelined, "value": B / (ms_pipelined * 1e-3),
+            "frac_of_hbm_peak": alg_bytes / (ms_pipelined * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "what": "same steps, sampler of batch i+1 on a second stream during gather i"},
         "step_GBps": alg_bytes / (ms_per_step * 1e-3) / 1e9,
         "step_frac_of_hbm_peak": alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": achieved,
@@ -525,6 +528,8 @@ def main():
     ap.add_argument("--trajectories5", type=int, default=2000,
                     help="config 5: trajectories of 1000 steps in pinned host memory (2000 = 56.5 GB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-pipelined", action="store_true",
+                    help="config 4: skip the second, pipelined pass over the same steps")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB plain copies (slices kernel) before the steps")
     ap.add_argument("--traffic-bytes", type=float, default=None,

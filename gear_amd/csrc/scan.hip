@@ -53,9 +53,20 @@ template <> struct OutVec2<float> {
 // non-temporal stores only reach full bandwidth when a wave writes whole cache lines.  With
 // 16 bytes per lane the lanes already do; with 32 bytes per lane (fp64 results of a float4) the
 // slice takes a detour through a wave-private LDS row.
+// Results that fit the caches are stored normally (the search that follows reads them back);
+// larger ones stream past the caches with non-temporal stores.
+template <typename V>
+__device__ __forceinline__ void store_vec(V *p, V v, bool nt) {
+  if (nt)
+    __builtin_nontemporal_store(v, p);
+  else
+    *p = v;
+}
+
 template <typename Out, int VE>
 __device__ __forceinline__ void store_slice(Out *__restrict__ out, int64_t e_wave, int64_t n,
                                             const Out (&v)[VE], Out *stage_row, int lane) {
+  const bool nt = n * (int64_t)sizeof(Out) > (32ll << 20);
   typedef typename OutVec2<Out>::type out_vec2;
   constexpr int kLaneBytes = VE * (int)sizeof(Out);
   const int64_t e0 = e_wave + (int64_t)lane * VE;
@@ -71,7 +82,7 @@ __device__ __forceinline__ void store_slice(Out *__restrict__ out, int64_t e_wav
       out_vec2 o;
       o[0] = v[j];
       o[1] = v[j + 1];
-      __builtin_nontemporal_store(o, reinterpret_cast<out_vec2 *>(out + e0 + j));
+      store_vec(reinterpret_cast<out_vec2 *>(out + e0 + j), o, nt);
     }
   } else {
 #pragma unroll
@@ -84,8 +95,8 @@ __device__ __forceinline__ void store_slice(Out *__restrict__ out, int64_t e_wav
       out_vec2 o;
       o[0] = stage_row[h * 2 * kWave + 2 * lane];
       o[1] = stage_row[h * 2 * kWave + 2 * lane + 1];
-      __builtin_nontemporal_store(
-          o, reinterpret_cast<out_vec2 *>(out + e_wave + (int64_t)h * 2 * kWave + 2 * lane));
+      store_vec(reinterpret_cast<out_vec2 *>(out + e_wave + (int64_t)h * 2 * kWave + 2 * lane), o,
+                nt);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
