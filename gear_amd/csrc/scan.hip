@@ -38,14 +38,15 @@ template <> struct InVec<int64_t, 2> {
   typedef int64_t type __attribute__((ext_vector_type(2), aligned(8)));
 };
 template <typename Acc> struct OutVec2;
+// result vectors are stored with their natural alignment (the launcher checks the pointer)
 template <> struct OutVec2<double> {
-  typedef double type __attribute__((ext_vector_type(2), aligned(8)));
+  typedef double type __attribute__((ext_vector_type(2)));
 };
 template <> struct OutVec2<int64_t> {
-  typedef int64_t type __attribute__((ext_vector_type(2), aligned(8)));
+  typedef int64_t type __attribute__((ext_vector_type(2)));
 };
 template <> struct OutVec2<float> {
-  typedef float type __attribute__((ext_vector_type(2), aligned(4)));
+  typedef float type __attribute__((ext_vector_type(2)));
 };
 
 // Writes the VE consecutive results of every lane of a wave (a contiguous slice of 64*VE
@@ -387,7 +388,7 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
   if (!ws || ws_bytes < scan_ws_bytes(n) || (reinterpret_cast<uintptr_t>(ws) & 7))
     return GEAR_HIP_EWORKSPACE;
   if ((reinterpret_cast<uintptr_t>(in) & (sizeof(In) - 1)) ||
-      (reinterpret_cast<uintptr_t>(out) & (sizeof(Out) - 1)))
+      (reinterpret_cast<uintptr_t>(out) & 15))
     return GEAR_HIP_EALIGN;
   // few enough ranges: no look-back chain (4, 8 or 16 rows of 256 vectors per workgroup)
   const int64_t row = (int64_t)kBlock * VE;

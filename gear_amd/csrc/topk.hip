@@ -19,11 +19,10 @@ constexpr int kHistBins = 2048;
 constexpr int kMaxHistBlocks = 512;
 
 struct State {
-  uint32_t prefix;   // key bits decided so far (right-aligned)
-  uint32_t k_rem;    // entries still to take from the bin being refined
-  uint32_t done[3];  // finished workgroups per histogram pass
-  uint32_t ticket;   // tile ticket of the compaction pass
-  uint32_t pad[58];
+  uint32_t prefix[3];  // key bits decided after pass 0, 1, 2 (right-aligned)
+  uint32_t k_rem[3];   // entries still to take from the bin picked in that pass
+  uint32_t ticket;     // tile ticket of the compaction pass
+  uint32_t pad[57];
 };
 static_assert(sizeof(State) == 256, "State is the 256-byte header of the workspace");
 
@@ -60,22 +59,71 @@ __global__ void zero_kernel(uint32_t *p, int64_t words) {
   if (i < words) p[i] = 0u;
 }
 
+// Every thread of a 256-thread workgroup calls this: walk the histogram of pass PASS from the top
+// bin down and stop at the bin that holds the k_rem-th largest remaining key.  The result
+// (key prefix after this pass, entries still needed inside that bin) is returned to all threads.
+// The kernel that needs the result computes it itself instead of waiting for a launch of its own;
+// workgroup 0 also records it in `state` for the kernels after it.
+struct Pick {
+  uint32_t prefix, k_rem;
+};
+template <int PASS>
+__device__ __forceinline__ Pick pick_bin(int64_t k, State *state, const uint32_t *hist) {
+  constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
+  constexpr int kPerThread = kBinsHere / kBlock;
+  __shared__ uint32_t wsum[kBlock / kWave];
+  __shared__ Pick s_pick;
+  const int tid = threadIdx.x;
+  const uint32_t prefix = PASS == 0 ? 0u : state->prefix[PASS == 0 ? 0 : PASS - 1];
+  const uint32_t k_rem = PASS == 0 ? (uint32_t)k : state->k_rem[PASS == 0 ? 0 : PASS - 1];
+  // thread t owns bins top-down: kBinsHere-1 - t*kPerThread - j
+  uint32_t c[kPerThread];
+  int tsum = 0;
+#pragma unroll
+  for (int j = 0; j < kPerThread; ++j) {
+    c[j] = hist[kBinsHere - 1 - tid * kPerThread - j];
+    tsum += (int)c[j];
+  }
+  const int inc = wave_inclusive_sum(tsum);
+  if ((tid & 63) == 63) wsum[tid >> 6] = (uint32_t)inc;
+  __syncthreads();
+  uint32_t running = (uint32_t)(inc - tsum);
+  for (int w = 0; w < (tid >> 6); ++w) running += wsum[w];
+#pragma unroll
+  for (int j = 0; j < kPerThread; ++j) {
+    if (running < k_rem && running + c[j] >= k_rem) {
+      const uint32_t bin = (uint32_t)(kBinsHere - 1 - tid * kPerThread - j);
+      s_pick.prefix = PASS == 0 ? bin : (PASS == 1 ? ((prefix << 11) | bin) : ((prefix << 10) | bin));
+      s_pick.k_rem = k_rem - running;
+    }
+    running += c[j];
+  }
+  __syncthreads();
+  const Pick r = s_pick;
+  if (blockIdx.x == 0 && tid == 0) {
+    state->prefix[PASS] = r.prefix;
+    state->k_rem[PASS] = r.k_rem;
+  }
+  return r;
+}
+
 // PASS 0: bits 31..21, PASS 1: bits 20..10 of keys whose top 11 bits equal state->prefix,
 // PASS 2: bits 9..0 of keys whose top 22 bits equal state->prefix.  Workgroups count into LDS and
-// add their non-empty bins to the global histogram; the bin is picked by select_pick_kernel in a
-// launch of its own (a device-scope fence per workgroup for a "last workgroup picks" scheme costs
-// far more on this multi-XCD part than one small launch).
+// add their non-empty bins to the global histogram of this pass (hist; the previous pass's is
+// at hist - kHistBins); the bin of the previous pass is picked by every workgroup for itself.
 template <int PASS>
 __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__restrict__ p,
-                                                             int64_t n, const State *state,
+                                                             int64_t n, int64_t k, State *state,
                                                              uint32_t *hist) {
   constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
   typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
   __shared__ uint32_t h[kBinsHere];
   const int tid = threadIdx.x;
   for (int i = tid; i < kBinsHere; i += kBlock) h[i] = 0;
+  uint32_t prefix = 0u;
+  if (PASS == 1) prefix = pick_bin<0>(k, state, hist - kHistBins).prefix;
+  if (PASS == 2) prefix = pick_bin<1>(k, state, hist - kHistBins).prefix;
   __syncthreads();
-  const uint32_t prefix = PASS == 0 ? 0u : state->prefix;
 
   auto count = [&](float f) {
     const uint32_t key = order_key(f);
@@ -101,41 +149,6 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__rest
     if (h[i]) atomicAdd(&hist[i], h[i]);
 }
 
-// One workgroup: walk the histogram from the top bin down and stop at the bin that holds the
-// k_rem-th largest remaining key.
-template <int PASS>
-__global__ __launch_bounds__(kBlock) void select_pick_kernel(int64_t k, State *state,
-                                                             const uint32_t *hist) {
-  constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
-  constexpr int kPerThread = kBinsHere / kBlock;
-  __shared__ uint32_t wsum[kBlock / kWave];
-  const int tid = threadIdx.x;
-  const uint32_t prefix = PASS == 0 ? 0u : state->prefix;
-  const uint32_t k_rem = PASS == 0 ? (uint32_t)k : state->k_rem;
-  // thread t owns bins top-down: kBinsHere-1 - t*kPerThread - j
-  uint32_t c[kPerThread];
-  int tsum = 0;
-#pragma unroll
-  for (int j = 0; j < kPerThread; ++j) {
-    c[j] = hist[kBinsHere - 1 - tid * kPerThread - j];
-    tsum += (int)c[j];
-  }
-  const int inc = wave_inclusive_sum(tsum);
-  if ((tid & 63) == 63) wsum[tid >> 6] = (uint32_t)inc;
-  __syncthreads();
-  uint32_t running = (uint32_t)(inc - tsum);
-  for (int w = 0; w < (tid >> 6); ++w) running += wsum[w];
-#pragma unroll
-  for (int j = 0; j < kPerThread; ++j) {
-    if (running < k_rem && running + c[j] >= k_rem) {
-      const uint32_t bin = (uint32_t)(kBinsHere - 1 - tid * kPerThread - j);
-      state->prefix = PASS == 0 ? bin : (PASS == 1 ? ((prefix << 11) | bin) : ((prefix << 10) | bin));
-      state->k_rem = k_rem - running;
-    }
-    running += c[j];
-  }
-}
-
 // packed per-tile descriptor: status (2 bits) | greater (31 bits) | equal (31 bits)
 constexpr uint64_t kStatusAggregate = 1ull << 62;
 constexpr uint64_t kStatusInclusive = 2ull << 62;
@@ -143,7 +156,8 @@ constexpr uint64_t kCountMask = (1ull << 62) - 1;
 
 template <bool DIRECT>
 __global__ __launch_bounds__(kBlock) void compact_kernel(
-    const float *__restrict__ p, int64_t n, State *state, uint64_t *desc,
+    const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist2,
+    uint64_t *desc,
     uint32_t *__restrict__ ckey, uint32_t *__restrict__ cidx, float *__restrict__ values_out,
     int64_t *__restrict__ indices_out) {
   typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -156,8 +170,9 @@ __global__ __launch_bounds__(kBlock) void compact_kernel(
   __syncthreads();
   const int64_t tile = s_tile;
   const int64_t base = tile * kTile;
-  const uint32_t thr = state->prefix;
-  const uint32_t need_eq = state->k_rem;
+  const Pick pk = pick_bin<2>(k, state, hist2);
+  const uint32_t thr = pk.prefix;
+  const uint32_t need_eq = pk.k_rem;
 
   uint32_t key[kRows][4];
   int s[kRows];  // packed counts of the thread's vector: greater << 16 | equal
@@ -269,7 +284,8 @@ constexpr uint64_t kRangeReady = 1ull << 63;
 
 template <bool DIRECT, int NR>
 __global__ __launch_bounds__(kBlock) void compact_ranges_kernel(
-    const float *__restrict__ p, int64_t n, State *state, uint64_t *desc,
+    const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist2,
+    uint64_t *desc,
     uint32_t *__restrict__ ckey, uint32_t *__restrict__ cidx, float *__restrict__ values_out,
     int64_t *__restrict__ indices_out) {
   typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -283,8 +299,9 @@ __global__ __launch_bounds__(kBlock) void compact_ranges_kernel(
   __syncthreads();
   const int64_t tile = s_tile;
   const int64_t base = tile * kElems;
-  const uint32_t thr = state->prefix;
-  const uint32_t need_eq = state->k_rem;
+  const Pick pk = pick_bin<2>(k, state, hist2);
+  const uint32_t thr = pk.prefix;
+  const uint32_t need_eq = pk.k_rem;
 
   float q[NR][4];
 #pragma unroll
@@ -417,13 +434,10 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   int64_t hblocks = ceil_div64(n, (int64_t)kBlock * 4 * 4);
   if (hblocks < 1) hblocks = 1;
   if (hblocks > kMaxHistBlocks) hblocks = kMaxHistBlocks;
-  const dim3 hgrid((unsigned)hblocks), block(kBlock), one(1);
-  select_hist_kernel<0><<<hgrid, block, 0, st>>>(priorities, n, state, hist);
-  select_pick_kernel<0><<<one, block, 0, st>>>(k, state, hist);
-  select_hist_kernel<1><<<hgrid, block, 0, st>>>(priorities, n, state, hist + kHistBins);
-  select_pick_kernel<1><<<one, block, 0, st>>>(k, state, hist + kHistBins);
-  select_hist_kernel<2><<<hgrid, block, 0, st>>>(priorities, n, state, hist + 2 * kHistBins);
-  select_pick_kernel<2><<<one, block, 0, st>>>(k, state, hist + 2 * kHistBins);
+  const dim3 hgrid((unsigned)hblocks), block(kBlock);
+  select_hist_kernel<0><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist);
+  select_hist_kernel<1><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist + kHistBins);
+  select_hist_kernel<2><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
 
   uint32_t *ckey = reinterpret_cast<uint32_t *>(ws + l.ckey);
@@ -434,11 +448,11 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   do {                                                                                          \
     const unsigned g = (unsigned)ceil_div64(n, (NR) * row);                                     \
     if (direct)                                                                                 \
-      compact_ranges_kernel<true, NR><<<dim3(g), block, 0, st>>>(priorities, n, state, desc,    \
+      compact_ranges_kernel<true, NR><<<dim3(g), block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins, desc,    \
                                                                  ckey, cidx, values_out,        \
                                                                  indices_out);                  \
     else                                                                                        \
-      compact_ranges_kernel<false, NR><<<dim3(g), block, 0, st>>>(priorities, n, state, desc,   \
+      compact_ranges_kernel<false, NR><<<dim3(g), block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins, desc,   \
                                                                   ckey, cidx, values_out,       \
                                                                   indices_out);                 \
   } while (0)
@@ -451,10 +465,10 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   } else {
     const int64_t tiles = ceil_div64(n, kTile);
     if (direct)
-      compact_kernel<true><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, state, desc, ckey,
+      compact_kernel<true><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins, desc, ckey,
                                                                     cidx, values_out, indices_out);
     else
-      compact_kernel<false><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, state, desc,
+      compact_kernel<false><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins, desc,
                                                                      ckey, cidx, values_out,
                                                                      indices_out);
   }

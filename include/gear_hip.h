@@ -171,7 +171,7 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
  * :276-278), which is fp32 and only correct for one block.
  * workspace: device memory of at least gear_hip_scan_workspace_bytes(n) bytes, 256-byte aligned;
  * its contents need not be initialised (the call initialises it on `stream`).
- * n may be 0 (nothing is written).  n <= 2^40. */
+ * n may be 0 (nothing is written).  n <= 2^40.  `out` must be 16-byte aligned. */
 size_t gear_hip_scan_workspace_bytes(int64_t n);
 int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspace,
                           size_t workspace_bytes, void *stream);
