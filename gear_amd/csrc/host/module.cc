@@ -63,10 +63,11 @@ void *current_stream() {
   return reinterpret_cast<void *>(s.attr("cuda_stream").cast<uintptr_t>());
 }
 
-// Device scratch owned by the module, grown on demand and kept (the C ABI itself never allocates).
-void *workspace(const char *tag, size_t bytes, size_t *have) {
-  static std::map<std::string, std::pair<void *, size_t>> cache;
-  auto &e = cache[tag];
+// Device scratch owned by the module, one per (purpose, stream), grown on demand and kept (the
+// C ABI itself never allocates; calls on different streams must not share a workspace).
+void *workspace(const char *tag, void *stream, size_t bytes, size_t *have) {
+  static std::map<std::pair<std::string, void *>, std::pair<void *, size_t>> cache;
+  auto &e = cache[std::make_pair(std::string(tag), stream)];
   if (e.second < bytes) {
     if (e.first) gear_hip_device_free(e.first);
     e.first = nullptr;
@@ -622,24 +623,26 @@ PYBIND11_MODULE(_libgear, libgear) {
         [](const py::object &val, const py::object &out, int) {
           TensorInfo v = tensor_info(val, "val", 4, 1), o = tensor_info(out, "out", 4, 1);
           size_t have = 0;
-          void *ws = workspace("sum", gear_hip_sum_workspace_bytes(v.numel), &have);
+          void *st = current_stream();
+          void *ws = workspace("sum", st, gear_hip_sum_workspace_bytes(v.numel), &have);
           check_hip("sum", gear_hip_sum_f32(static_cast<const float *>(v.ptr), v.numel,
-                                            static_cast<float *>(o.ptr), nullptr, ws, have, current_stream()));
+                                            static_cast<float *>(o.ptr), nullptr, ws, have, st));
         },
         py::arg("val"), py::arg("out"), py::arg("stride") = 1);
   m.def("prefix_sum", [](const py::object &input, const py::object &output) {
     TensorInfo in = tensor_info(input, "input", 4, 1), out = tensor_info(output, "output", 0, 1);
     if (out.numel < in.numel) throw std::runtime_error("output is shorter than input");
     size_t have = 0;
-    void *ws = workspace("scan", gear_hip_scan_workspace_bytes(in.numel), &have);
+    void *st = current_stream();
+    void *ws = workspace("scan", st, gear_hip_scan_workspace_bytes(in.numel), &have);
     if (out.elem == 8)
       check_hip("prefix_sum", gear_hip_scan_f32_f64(static_cast<const float *>(in.ptr),
                                                     static_cast<double *>(out.ptr), in.numel, ws, have,
-                                                    current_stream()));
+                                                    st));
     else if (out.elem == 4)
       check_hip("prefix_sum", gear_hip_scan_f32_f32(static_cast<const float *>(in.ptr),
                                                     static_cast<float *>(out.ptr), in.numel, ws, have,
-                                                    current_stream()));
+                                                    st));
     else
       throw std::runtime_error("output must be a float32 or float64 tensor");
   });

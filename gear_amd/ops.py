@@ -46,13 +46,14 @@ def _src_ptr(src):
 
 
 class _Workspace:
-    """Per-device scratch tensors, grown on demand and reused (no allocation in steady state)."""
+    """Scratch tensors per (purpose, device, stream), grown on demand and reused: no allocation
+    in steady state, and calls enqueued on different streams never share a workspace."""
 
     def __init__(self):
         self._bufs = {}
 
     def get(self, tag, nbytes, device):
-        key = (tag, device)
+        key = (tag, device, torch.cuda.current_stream(device).cuda_stream)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
