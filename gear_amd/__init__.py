@@ -42,4 +42,8 @@ def install_as_gear():
         mod = importlib.import_module(__name__ + "." + sub)
         sys.modules.setdefault("gear." + sub, mod)
         setattr(me, sub, mod)
+    # modules that pickled objects of the reference name (SharedDatasetMeta, IndexMeta)
+    for sub in ("dataset.shared_dataset", "sampler.global_sampler", "loader.offline_loader",
+                "loader.basic_loader"):
+        sys.modules.setdefault("gear." + sub, importlib.import_module(__name__ + "." + sub))
     return me

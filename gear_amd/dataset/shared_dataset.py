@@ -19,6 +19,15 @@ from ..utils import ensure_path, get_local_node_hashed_int32
 SharedDatasetMeta = namedtuple("SharedDatasetMeta", ["storage", "index"])
 IndexMeta = namedtuple("IndexMeta",
                        ["global_capacity", "local_capacity", "index_offset", "shared", "key"])
+# checkpoints name these two as the reference does (gear/dataset/shared_dataset.py:15-18)
+SharedDatasetMeta.__module__ = "gear.dataset.shared_dataset"
+IndexMeta.__module__ = "gear.dataset.shared_dataset"
+
+
+def _reference_module_names():
+    """Checkpoints refer to classes by the reference's module paths; make those resolvable."""
+    import gear_amd
+    gear_amd.install_as_gear()
 
 
 def _keys(key):
@@ -120,6 +129,7 @@ class SharedDataset(torch.utils.data.Dataset):
         """Three pickles in one file: meta, the table (spec, key, size, create, bytes), the index
         state (offset, local, global, timesteps||weights), as in shared_dataset.py:179-201."""
         ensure_path(path)
+        _reference_module_names()
         with open(path, "wb") as of:
             pickler = pickle.Pickler(of)
             pickler.dump(SharedDatasetMeta(
@@ -133,6 +143,7 @@ class SharedDataset(torch.utils.data.Dataset):
              create: bool = True, proc_rank: int = 0):
         self._table = None
         self._iset = None
+        _reference_module_names()
         table_key, iset_key = _keys(key)
         with open(pathlib.Path(path), "rb") as f:
             unpickler = pickle.Unpickler(f)

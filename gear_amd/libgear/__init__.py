@@ -21,4 +21,25 @@ comm = _libgear.comm
 _sys.modules[__name__ + ".core"] = core
 _sys.modules[__name__ + ".comm"] = comm
 
+# Pickles written by the reference name its classes `libgear.core.<Class>`
+# (src/storage/pybind.cc:28-40,53-69,85-99,178-204; src/index/pybind.cc:299-306).  The classes here
+# carry the same module path and the same state tuples, so checkpoints travel in both directions;
+# the names `libgear`, `libgear.core` resolve to this package unless a real `libgear` is installed.
+for _name in dir(core):
+    _obj = getattr(core, _name)
+    if isinstance(_obj, type):
+        try:
+            _obj.__module__ = "libgear.core"
+        except (AttributeError, TypeError):
+            pass
+        for _inner in vars(_obj).values():
+            if isinstance(_inner, type):
+                try:
+                    _inner.__module__ = "libgear.core"
+                except (AttributeError, TypeError):
+                    pass
+_sys.modules.setdefault("libgear", _sys.modules[__name__])
+_sys.modules.setdefault("libgear.core", core)
+_sys.modules.setdefault("libgear.comm", comm)
+
 __all__ = ["core", "comm"]

@@ -223,3 +223,64 @@ def test_multi_rank_entry_points_refuse():
         h.connect(0, 2, b"x")
     with pytest.raises(RuntimeError, match="single-GPU"):
         h.subsend(1)
+
+
+def test_checkpoint_stream_uses_reference_class_paths(tmp_path):
+    """A checkpoint names `libgear.core.*` / `gear.dataset.shared_dataset.*` classes with the
+    reference's state tuples (storage/pybind.cc:178-204, index/pybind.cc:15-50), so files written
+    by either side unpickle on the other; a stream assembled by hand from those tuples loads."""
+    import pickletools
+    from gear_amd.dataset import SharedDataset
+    gear_amd.install_as_gear()
+    tspec = TableSpec.create(trajectory_length=4, capacity=3,
+                             column_specs=[{"shape": [2], "dtype": torch.float32, "name": "x"}])
+    ds = SharedDataset.create(tspec, key=4242, placement="host")
+    for i in range(3):
+        ds[i] = (1.0 + i, i + 1, [torch.full((4, 2), float(i))])
+    path = tmp_path / "ref_style.pt"
+    ds.checkpoint(path)
+    names = set()
+    with open(path, "rb") as f:
+        data = f.read()
+    for op, arg, _ in pickletools.genops(data):
+        if op.name in ("GLOBAL", "STACK_GLOBAL") and arg:
+            names.add(arg)
+        if op.name in ("SHORT_BINUNICODE", "BINUNICODE") and isinstance(arg, str) and (
+                arg.startswith("libgear") or arg.startswith("gear")):
+            names.add(arg)
+    assert "libgear.core" in names and "gear.dataset.shared_dataset" in names
+    assert not any(n.startswith("gear_amd") for n in names)
+
+    # hand-built stream in the reference's layout: meta, table 5-tuple, index-state 4-tuple
+    import io
+    table_bytes = np.arange(tspec.size(), dtype=np.uint8)
+    ts = np.array([4, 3, 2], np.int64)
+    w = np.array([0.5, 0.25, 2.0], np.float32)
+    blob = np.concatenate([ts.view(np.uint8), w.view(np.uint8)])
+
+    def from_state(cls, state):              # what unpickling does: __new__, then __setstate__
+        obj = cls.__new__(cls)
+        obj.__setstate__(state)
+        return obj
+
+    from gear_amd.dataset.shared_dataset import IndexMeta, SharedDatasetMeta
+    os.environ["GEAR_TABLE_PLACEMENT"] = "host"
+    try:
+        table = from_state(glibc.TrajectoryTable, (tspec, 1234, int(tspec.size()), True, table_bytes))
+    finally:
+        del os.environ["GEAR_TABLE_PLACEMENT"]
+    state = from_state(glibc.IndexsetState, (0, 3, 3, blob))
+    buf = io.BytesIO()
+    pk = pkl.Pickler(buf, protocol=2)
+    pk.dump(SharedDatasetMeta(tspec, IndexMeta(3, 3, 0, False, 99)))
+    pk.dump(table)
+    pk.dump(state)
+    p2 = tmp_path / "handmade.pt"
+    p2.write_bytes(buf.getvalue())
+    os.environ["GEAR_TABLE_PLACEMENT"] = "host"
+    try:
+        loaded = SharedDataset().load(p2, key=777)
+    finally:
+        del os.environ["GEAR_TABLE_PLACEMENT"]
+    assert loaded.timesteps.tolist() == [4, 3, 2] and loaded.weights.tolist() == [0.5, 0.25, 2.0]
+    assert loaded._handler.raw(0, int(tspec.size())).tensor().tolist() == table_bytes.tolist()
