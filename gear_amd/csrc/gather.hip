@@ -18,21 +18,13 @@
 namespace gearhip {
 namespace {
 
-#ifndef GEARHIP_GATHER_BLOCK
-#define GEARHIP_GATHER_BLOCK 128
-#endif
-constexpr int kBlock = GEARHIP_GATHER_BLOCK;
-#ifndef GEARHIP_GATHER_TG_MAX_SHIFT
-#define GEARHIP_GATHER_TG_MAX_SHIFT 7
-#endif
+constexpr int kBlock = 128;       // threads per workgroup
+constexpr int kMaxGroupShift = 7;  // a group never spans workgroups: at most 128 threads
 
 enum GatherMode { kSubcopy = 0, kVcopy = 1, kCopy = 2 };
 
-#ifdef GEARHIP_GATHER_ADJ
-#define GEARHIP_VEC_INDEX(k0, u, tg, lane, U) ((k0) + (int64_t)(lane) * (U) + (u))
-#else
+// vector u of a lane: lanes of a group take consecutive vectors (coalesced 1 KiB per wave)
 #define GEARHIP_VEC_INDEX(k0, u, tg, lane, U) ((k0) + (int64_t)(u) * (tg) + (lane))
-#endif
 
 struct ColumnArgs {
   uint8_t *dst;
@@ -210,13 +202,7 @@ template <int U, int NT>
 __global__ __launch_bounds__(kBlock) void subcopy_multi_kernel(GatherArgs p, MultiArgs m) {
   // columns are laid out one after another along the grid; find this block's column
   int ci = 0;
-#ifdef GEARHIP_GATHER_XCD
-  const int64_t per = (gridDim.x + 7) / 8;
-  int64_t b = (int64_t)(blockIdx.x & 7) * per + (blockIdx.x >> 3);
-  if (b >= gridDim.x) return;
-#else
   const int64_t b = blockIdx.x;
-#endif
 #pragma unroll 1
   for (int i = 1; i < m.ncols; ++i)
     if (b >= m.col[i].block_begin) ci = i;
@@ -312,7 +298,7 @@ Shape plan(int64_t num, int64_t max_region, int U) {
   if (nvec < 1) nvec = 1;
   int64_t want = ceil_div64(nvec, U);
   int sh = 0;
-  while ((1ll << sh) < want && sh < GEARHIP_GATHER_TG_MAX_SHIFT) ++sh;
+  while ((1ll << sh) < want && sh < kMaxGroupShift) ++sh;
   s.tg_shift = sh;
   s.cps = ceil_div64(nvec, (int64_t)U << sh);
   const int64_t threads = num * s.cps * (1ll << sh);

@@ -392,10 +392,6 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
     return GEAR_HIP_EALIGN;
   // few enough ranges: no look-back chain (4, 8 or 16 rows of 256 vectors per workgroup)
   const int64_t row = (int64_t)kBlock * VE;
-  static const int force_nr = env_int("GEAR_HIP_SCAN_ROWS", 0);  // experiments only
-  if (force_nr == 4) return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st);
-  if (force_nr == 8) return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st);
-  if (force_nr == 16) return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st);
   if (ceil_div64(n, 4 * row) <= 1024) return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st);
   if (ceil_div64(n, 8 * row) <= 1024) return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st);
   if (ceil_div64(n, 16 * row) <= kMaxRanges)
