@@ -13,6 +13,7 @@
 
 #include "gear_hip.h"
 #include "indexset.hpp"
+#include "requests.hpp"
 #include "storage.hpp"
 
 namespace py = pybind11;
@@ -588,6 +589,51 @@ PYBIND11_MODULE(_libgear, libgear) {
       .def_property_readonly("device_weights_address",
                              [](const Indexset &s) { return reinterpret_cast<uintptr_t>(s.device_weights()); })
       .def("get_state", [](Indexset &s) { return std::make_shared<IndexsetState>(s.get_state()); });
+
+  // ---- request arrays of the online path (src/index/pybind.cc:154-206) -------------------------
+  py::class_<InferenceRequestArray>(m, "InferenceRequestArray")
+      .def_readonly("count", &InferenceRequestArray::count)
+      .def("insert", &InferenceRequestArray::insert)
+      .def("clear", &InferenceRequestArray::clear)
+      .def("source_element_view", [](InferenceRequestArray &a, size_t i) { return a.srcs[i]; })
+      .def("index_element_view", [](InferenceRequestArray &a, size_t i) { return a.idxs[i]; })
+      .def("timestep_element_view", [](InferenceRequestArray &a, size_t i) { return a.tss[i]; })
+      .def("source_tensor_view",
+           [](InferenceRequestArray &a) {
+             SpanBase s;
+             s.ptr = a.srcs;
+             return span_to_tensor(s, (int64_t)a.count * 4, DataType::kInt32);
+           }, py::keep_alive<0, 1>())
+      .def("index_tensor_view",
+           [](InferenceRequestArray &a) {
+             SpanBase s;
+             s.ptr = a.idxs;
+             return span_to_tensor(s, (int64_t)a.count * 8, DataType::kInt64);
+           }, py::keep_alive<0, 1>())
+      .def("timestep_tensor_view",
+           [](InferenceRequestArray &a) {
+             SpanBase s;
+             s.ptr = a.tss;
+             return span_to_tensor(s, (int64_t)a.count * 8, DataType::kInt64);
+           }, py::keep_alive<0, 1>());
+
+  py::class_<WeightUpdateRequestArray>(m, "WeightUpdateRequestArray")
+      .def_readonly("count", &WeightUpdateRequestArray::count)
+      .def("update", &WeightUpdateRequestArray::update)
+      .def("updated_element_view", [](WeightUpdateRequestArray &a, size_t i) { return a.updated.at(i) != 0; })
+      .def("timestep_element_view", [](WeightUpdateRequestArray &a, size_t i) { return a.timesteps[i]; })
+      .def("weight_element_view", [](WeightUpdateRequestArray &a, size_t i) { return a.weights[i]; });
+
+  py::class_<CachedRequest, std::shared_ptr<CachedRequest>>(m, "CachedRequest")
+      .def(py::init<int64_t>())
+      .def_readonly("capacity", &CachedRequest::capacity)
+      .def_readonly("iarr", &CachedRequest::iarr)
+      .def_readonly("warr", &CachedRequest::warr)
+      .def("continuous", [](CachedRequest &self, const py::object &idxs, const py::object &weights) {
+        TensorInfo a = tensor_info(idxs, "idxs", 8, 0), b = tensor_info(weights, "weights", 4, 0);
+        return self.warr.continuous(static_cast<int64_t *>(a.ptr), a.numel,
+                                    static_cast<float *>(b.ptr), b.numel);
+      });
 
   // ---- kernel launchers (src/cuda/*.cu tails) ----------------------------------------------------
   m.def("init", [](int device_id) { check_hip("init", gear_hip_set_device(device_id)); });

@@ -10,9 +10,10 @@ namespace {
 
 constexpr int kBlock = 256;
 
-__global__ __launch_bounds__(kBlock) void scatter_unique_kernel(float *__restrict__ w, int64_t n,
+template <typename T>
+__global__ __launch_bounds__(kBlock) void scatter_unique_kernel(T *__restrict__ w, int64_t n,
                                                                 const int64_t *__restrict__ idx,
-                                                                const float *__restrict__ v,
+                                                                const T *__restrict__ v,
                                                                 int64_t num) {
   const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (j >= num) return;
@@ -31,10 +32,11 @@ __global__ __launch_bounds__(kBlock) void scatter_prepare_kernel(const int64_t *
   pos[j] = (uint32_t)j;
 }
 
-__global__ __launch_bounds__(kBlock) void scatter_winners_kernel(float *__restrict__ w, int64_t n,
+template <typename T>
+__global__ __launch_bounds__(kBlock) void scatter_winners_kernel(T *__restrict__ w, int64_t n,
                                                                  const uint64_t *__restrict__ keys,
                                                                  const uint32_t *__restrict__ pos,
-                                                                 const float *__restrict__ v,
+                                                                 const T *__restrict__ v,
                                                                  int64_t num) {
   const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (j >= num) return;
@@ -70,9 +72,10 @@ using namespace gearhip;
 
 extern "C" size_t gear_hip_scatter_workspace_bytes(int64_t num) { return layout(num).total; }
 
-extern "C" int gear_hip_scatter_f32(float *weights, int64_t n, const int64_t *idx,
-                                    const float *values, int64_t num, int unique_indices,
-                                    void *workspace, size_t workspace_bytes, void *stream) {
+namespace {
+template <typename T>
+int scatter_any(T *weights, int64_t n, const int64_t *idx, const T *values, int64_t num,
+                int unique_indices, void *workspace, size_t workspace_bytes, void *stream) {
   if (n < 0 || num < 0) return GEAR_HIP_EINVAL;
   if (num == 0 || n == 0) return 0;
   if (!weights || !idx || !values) return GEAR_HIP_EINVAL;
@@ -80,7 +83,7 @@ extern "C" int gear_hip_scatter_f32(float *weights, int64_t n, const int64_t *id
   hipStream_t st = as_stream(stream);
   const dim3 grid((unsigned)ceil_div64(num, kBlock)), block(kBlock);
   if (unique_indices) {
-    scatter_unique_kernel<<<grid, block, 0, st>>>(weights, n, idx, values, num);
+    scatter_unique_kernel<T><<<grid, block, 0, st>>>(weights, n, idx, values, num);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
@@ -101,7 +104,22 @@ extern "C" int gear_hip_scatter_f32(float *weights, int64_t n, const int64_t *id
       reinterpret_cast<uint32_t *>(ws + l.vtmp), num, 0, bits,
       reinterpret_cast<uint32_t *>(ws + l.hist), st);
   if (rc) return rc;
-  scatter_winners_kernel<<<grid, block, 0, st>>>(weights, n, kout, vout, values, num);
+  scatter_winners_kernel<T><<<grid, block, 0, st>>>(weights, n, kout, vout, values, num);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
+}
+}  // namespace
+
+extern "C" int gear_hip_scatter_f32(float *weights, int64_t n, const int64_t *idx,
+                                    const float *values, int64_t num, int unique_indices,
+                                    void *workspace, size_t workspace_bytes, void *stream) {
+  return scatter_any<float>(weights, n, idx, values, num, unique_indices, workspace,
+                            workspace_bytes, stream);
+}
+
+extern "C" int gear_hip_scatter_i64(int64_t *table, int64_t n, const int64_t *idx,
+                                    const int64_t *values, int64_t num, int unique_indices,
+                                    void *workspace, size_t workspace_bytes, void *stream) {
+  return scatter_any<int64_t>(table, n, idx, values, num, unique_indices, workspace,
+                              workspace_bytes, stream);
 }

@@ -98,6 +98,32 @@ class OfflineLoader(BasicLoader):
                     values.to(self._mpu.device, torch.float32).contiguous(),
                     unique_indices=unique_indices)
 
+    def apply_cached_updates(self, cache):
+        """Flush the pending weight updates of a CachedRequest (dedupe done on the host, last
+        write wins, src/index/request.cc:41-75) into the device priorities and lengths; the host
+        index set is updated too (what SharedMemoryIndexServer.update is meant to do,
+        src/index/server.cc:175-180).  Returns the number of updated trajectories."""
+        cap = cache.capacity
+        if not hasattr(self, "_upd_idx") or self._upd_idx.numel() < 2 * cap:
+            pin = torch.cuda.is_available()
+            self._upd_idx = torch.empty(2 * cap, dtype=torch.int64, pin_memory=pin)
+            self._upd_w = torch.empty(cap, dtype=torch.float32, pin_memory=pin)
+        num = cache.continuous(self._upd_idx, self._upd_w)
+        if num == 0:
+            return 0
+        idx = self._upd_idx[:num]
+        ts = self._upd_idx[cap:cap + num]
+        w = self._upd_w[:num]
+        local = idx - self._iset.index_offset if self._iset.index_offset else idx
+        self._iset.weights[local] = w
+        self._iset.timesteps[local] = ts
+        dev = self._mpu.device
+        didx = local.to(dev, non_blocking=True)
+        ops.scatter(self._device_weights, didx, w.to(dev, non_blocking=True), unique_indices=True)
+        ops.scatter(self._device_timesteps, didx, ts.to(dev, non_blocking=True),
+                    unique_indices=True)
+        return num
+
     @property
     def table_spec(self):
         return self._table.get_table_spec() if self._table else None

@@ -318,10 +318,12 @@ def topk(priorities, k, *, sorted_by_value=True, want_values=True):
 
 
 def scatter(weights, idx, values, *, unique_indices=False):
-    """weights[idx[j]] = values[j]; duplicates: last one wins."""
-    _need(weights, torch.float32, "weights")
+    """weights[idx[j]] = values[j]; duplicates: last one wins.  fp32 or int64 tables."""
+    if weights.dtype not in (torch.float32, torch.int64):
+        raise TypeError("scatter works on float32 or int64 tables")
+    _need(weights, weights.dtype, "weights")
     _need(idx, torch.int64, "idx")
-    _need(values, torch.float32, "values")
+    _need(values, weights.dtype, "values")
     num = idx.numel()
     if values.numel() != num:
         raise ValueError("idx and values differ in length")
@@ -329,6 +331,7 @@ def scatter(weights, idx, values, *, unique_indices=False):
     if not unique_indices:
         nbytes = load().gear_hip_scatter_workspace_bytes(num)
         ws = _ws.get("scatter", nbytes, weights.device)
-    call("gear_hip_scatter_f32", _ptr(weights), weights.numel(), _ptr(idx), _ptr(values), num,
+    fn = "gear_hip_scatter_f32" if weights.dtype == torch.float32 else "gear_hip_scatter_i64"
+    call(fn, _ptr(weights), weights.numel(), _ptr(idx), _ptr(values), num,
          int(bool(unique_indices)), _ptr(ws), ws.numel() if ws is not None else 0, _stream())
     return weights

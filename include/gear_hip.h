@@ -274,6 +274,13 @@ int gear_hip_scatter_f32(float *weights, int64_t n, const int64_t *idx, const fl
                          int64_t num, int unique_indices, void *workspace,
                          size_t workspace_bytes, void *stream);
 
+/* The same update for int64 tables: timesteps[idx[j]] = values[j] (the trajectory lengths that
+ * travel with the priorities in a weight-update request, src/index/server.cc:175-180,
+ * Indexset::set_timestep, include/index/set.h:242-244).  Same workspace query. */
+int gear_hip_scatter_i64(int64_t *table, int64_t n, const int64_t *idx, const int64_t *values,
+                         int64_t num, int unique_indices, void *workspace, size_t workspace_bytes,
+                         void *stream);
+
 #if defined(__GNUC__)
 #pragma GCC visibility pop
 #endif

@@ -230,3 +230,39 @@ def test_update_priorities_then_topk(oracle):
     expect = oracle.topk_f32(w, 8, False)[1]
     assert set([3, 7, 40]).issubset(set(expect.tolist()))
     assert timesteps.tolist() == [raw["len"][i] for i in expect]
+
+
+def test_cached_weight_updates_reach_the_device(oracle):
+    """Online path: pending updates (deduplicated on the host, last write wins) are scattered into
+    the device priorities and lengths, then sampled from."""
+    from gear_amd.libgear import core as glibc
+    from gear_amd.loader import OfflineLoader
+    ds, raw = _dataset("pinned", seed=9)
+    loader = OfflineLoader(ds, 8, _mpu(), "TopK", PATTERNS)
+    w = ds.weights.numpy().copy()
+    ts = ds.timesteps.numpy().copy()
+    cache = glibc.CachedRequest(48)
+    rng = np.random.default_rng(9)
+    for _ in range(100):
+        i = int(rng.integers(0, 48))
+        t = int(rng.integers(1, 41))
+        x = float(rng.random()) + 5.0
+        cache.warr.update(i, t, x)
+        w[i], ts[i] = np.float32(x), t
+    announce("apply cached weight updates")
+    n = loader.apply_cached_updates(cache)
+    torch.cuda.synchronize()
+    assert n == len(set(np.nonzero(w >= 5.0)[0].tolist()))
+    assert np.array_equal(loader._device_weights.cpu().numpy(), w)
+    assert np.array_equal(loader._device_timesteps.cpu().numpy(), ts)
+    assert np.array_equal(ds.weights.numpy(), w) and np.array_equal(ds.timesteps.numpy(), ts)
+    timesteps, _ = next(loader)
+    expect = oracle.topk_f32(w, 8, False)[1]
+    assert timesteps.tolist() == ts[expect].tolist()
+    # int64 scatter with duplicates: last write wins
+    from gear_amd import ops
+    tab = torch.zeros(100, dtype=torch.int64, device="cuda")
+    idx = torch.tensor([5, 7, 5, 99, 7, 5], device="cuda")
+    val = torch.tensor([1, 2, 3, 4, 5, 6], device="cuda")
+    ops.scatter(tab, idx, val, unique_indices=False)
+    assert tab[5].item() == 6 and tab[7].item() == 5 and tab[99].item() == 4

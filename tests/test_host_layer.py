@@ -284,3 +284,34 @@ def test_checkpoint_stream_uses_reference_class_paths(tmp_path):
         del os.environ["GEAR_TABLE_PLACEMENT"]
     assert loaded.timesteps.tolist() == [4, 3, 2] and loaded.weights.tolist() == [0.5, 0.25, 2.0]
     assert loaded._handler.raw(0, int(tspec.size())).tensor().tolist() == table_bytes.tolist()
+
+
+def test_weight_update_requests_dedupe_last_wins():
+    """request.cc:41-75: one pending update per index (the last one), in order of first
+    appearance; continuous() packs (index, timestep at +capacity, weight) and clears."""
+    cache = glibc.CachedRequest(16)
+    model = {}
+    order = []
+    rng = random.Random(3)
+    for _ in range(60):
+        i, ts, w = rng.randrange(16), rng.randrange(100), rng.random()
+        cache.warr.update(i, ts, w)
+        if i not in model:
+            order.append(i)
+        model[i] = (ts, np.float32(w))
+    assert cache.warr.count == len(order)
+    idxs = torch.zeros(32, dtype=torch.long)
+    weights = torch.zeros(16, dtype=torch.float32)
+    num = cache.continuous(idxs, weights)
+    assert num == len(order)
+    assert idxs[:num].tolist() == order
+    assert idxs[16:16 + num].tolist() == [model[i][0] for i in order]
+    assert weights[:num].tolist() == [float(model[i][1]) for i in order]
+    assert cache.warr.count == 0 and cache.continuous(idxs, weights) == 0
+    assert not any(cache.warr.updated_element_view(i) for i in range(16))
+    with pytest.raises(RuntimeError, match="less space"):
+        cache.warr.update(1, 1, 1.0)
+        cache.continuous(torch.zeros(3, dtype=torch.long), weights)
+    cache.iarr.insert(2, 7, 11)
+    assert cache.iarr.count == 1 and cache.iarr.index_element_view(0) == 7
+    assert cache.iarr.timestep_tensor_view().tolist() == [11]
