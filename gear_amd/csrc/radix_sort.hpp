@@ -1,10 +1,16 @@
 // Stable least-significant-digit radix sort (8-bit digits) for key/value pairs, gfx950.
 //
-// Per digit: (1) every tile counts its digits in an LDS histogram, (2) one workgroup turns the
-// digit-major table of tile counts into global offsets, (3) every tile re-reads its keys, ranks
-// them in LDS (wave ballots give the rank among equal digits inside a wave, a small LDS table
-// the rank across the waves of the tile) and scatters keys and payloads to their final place for
-// this digit.  Ranks follow element order, so the sort is stable.
+// Per digit every tile re-reads its keys, ranks them in LDS (wave ballots give the rank among equal
+// digits inside a wave, a small LDS table the rank across the waves of the tile) and scatters keys
+// and payloads to their final place for this digit.  Ranks follow element order, so the sort is
+// stable.  Where a key lands depends on a table of (tile, digit) counts:
+//  * up to kFusedTiles tiles (the candidate lists of top-k, index batches): one launch per digit.
+//    The table is tile-major; every workgroup sums the counts of the tiles before it and scans the
+//    digit totals itself, and while it scatters it counts the next digit of every key into the
+//    next table at the tile the key lands in (global atomics).  Three tables rotate: read, count,
+//    clear.  A first launch counts digit 0.
+//  * more tiles: count launch, one workgroup per digit scans its row of the digit-major table,
+//    scatter launch.
 #pragma once
 #include "wave.hpp"
 
@@ -15,11 +21,12 @@ namespace {  // every translation unit gets its own copy of the kernels
 constexpr int kBlock = 256;
 constexpr int kBins = 256;
 constexpr int kWaves = kBlock / kWave;
-constexpr int kScanBlock = 1024;
+constexpr int kFusedTiles = 128;
 
 struct Plan {
   int rounds;      // elements per thread and tile
   int64_t ntiles;  // tiles of kBlock * rounds elements
+  bool fused;      // one launch per digit
 };
 
 inline Plan plan(int64_t num) {
@@ -29,18 +36,25 @@ inline Plan plan(int64_t num) {
   if (r > 64) r = 64;
   p.rounds = (int)r;
   p.ntiles = num <= 0 ? 0 : ceil_div64(num, (int64_t)kBlock * r);
+  p.fused = p.ntiles <= kFusedTiles;
   return p;
 }
 
+inline size_t table_bytes(const Plan &p) { return (size_t)p.ntiles * kBins * sizeof(uint32_t); }
+
+// digit totals (1 KiB) followed by one table, or by three where the launches are fused
 inline size_t hist_bytes(int64_t num) {
-  return align_up((size_t)plan(num).ntiles * kBins * sizeof(uint32_t) + 256, 256);
+  const Plan p = plan(num);
+  return align_up(kBins * sizeof(uint32_t) + (p.fused ? 3 : 1) * table_bytes(p) + 256, 256);
 }
 
-template <typename K>
+// Counts the digit of every key of a tile.  TILE_MAJOR: hist[tile][digit] and the workgroup also
+// clears its row of `clear` (the table the first scatter launch counts into).
+template <typename K, bool TILE_MAJOR>
 __global__ __launch_bounds__(kBlock) void hist_kernel(const K *__restrict__ keys, int64_t num,
                                                       int shift, uint32_t dmask, int rounds,
-                                                      int64_t ntiles,
-                                                      uint32_t *__restrict__ hist) {
+                                                      int64_t ntiles, uint32_t *__restrict__ hist,
+                                                      uint32_t *__restrict__ clear) {
   __shared__ uint32_t h[kBins];
   const int tid = threadIdx.x;
   h[tid] = 0;
@@ -51,55 +65,97 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const K *__restrict__ keys
     if (i < num) atomicAdd(&h[(uint32_t)(keys[i] >> shift) & dmask], 1u);
   }
   __syncthreads();
-  hist[(int64_t)tid * ntiles + blockIdx.x] = h[tid];
+  if (TILE_MAJOR) {
+    hist[(int64_t)blockIdx.x * kBins + tid] = h[tid];
+    clear[(int64_t)blockIdx.x * kBins + tid] = 0u;
+  } else {
+    hist[(int64_t)tid * ntiles + blockIdx.x] = h[tid];
+  }
 }
 
-// Exclusive scan of m counters in place, one workgroup.
-__global__ __launch_bounds__(kScanBlock) void hist_scan_kernel(uint32_t *h, int64_t m) {
-  __shared__ uint32_t wsum[kScanBlock / kWave];
-  __shared__ uint32_t carry;
+// Workgroup d turns row d of the digit-major table into exclusive prefixes over the tiles and
+// records the row's total.
+__global__ __launch_bounds__(kBlock) void digit_scan_kernel(uint32_t *__restrict__ table,
+                                                            int64_t ntiles,
+                                                            uint32_t *__restrict__ totals) {
+  __shared__ uint32_t wsum[kWaves];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid == 0) carry = 0;
-  __syncthreads();
-  for (int64_t base = 0; base < m; base += kScanBlock) {
+  uint32_t *row = table + (int64_t)blockIdx.x * ntiles;
+  uint32_t carry = 0;
+  for (int64_t base = 0; base < ntiles; base += kBlock) {
     const int64_t i = base + tid;
-    const int v = i < m ? (int)h[i] : 0;
+    const int v = i < ntiles ? (int)row[i] : 0;
     const int inc = wave_inclusive_sum(v);
     if (lane == 63) wsum[wave] = (uint32_t)inc;
     __syncthreads();
     uint32_t before = carry, total = 0;
-    for (int w = 0; w < kScanBlock / kWave; ++w) {
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
       if (w < wave) before += wsum[w];
       total += wsum[w];
     }
-    if (i < m) h[i] = before + (uint32_t)(inc - v);
-    __syncthreads();
-    if (tid == 0) carry += total;
+    if (i < ntiles) row[i] = before + (uint32_t)(inc - v);
+    carry += total;
     __syncthreads();
   }
+  if (tid == 0) totals[blockIdx.x] = carry;
 }
 
-template <typename K, typename V, bool HAS_V>
-__global__ __launch_bounds__(kBlock) void scatter_kernel(const K *__restrict__ kin,
-                                                         const V *__restrict__ vin,
-                                                         K *__restrict__ kout,
-                                                         V *__restrict__ vout, int64_t num,
-                                                         int shift, uint32_t dmask, int rounds,
-                                                         int64_t ntiles,
-                                                         const uint32_t *__restrict__ offsets) {
+// FUSED: `table` holds this digit's raw tile-major counts, `next` (may be null on the last digit)
+// receives the counts of the next digit, `clear` (may be null) is zeroed for the launch after.
+// Otherwise `table` holds the digit-major row prefixes and `totals` the digit totals.
+template <typename K, typename V, bool HAS_V, bool FUSED>
+__global__ __launch_bounds__(kBlock) void scatter_kernel(
+    const K *__restrict__ kin, const V *__restrict__ vin, K *__restrict__ kout,
+    V *__restrict__ vout, int64_t num, int shift, uint32_t dmask, int rounds, int64_t ntiles,
+    const uint32_t *__restrict__ table, const uint32_t *__restrict__ totals,
+    uint32_t *__restrict__ next, int next_shift, uint32_t next_dmask,
+    uint32_t *__restrict__ clear) {
   __shared__ uint32_t base[kBins];
   __shared__ uint32_t wcnt[kWaves][kBins];
+  __shared__ uint32_t wsum[kWaves];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  base[tid] = offsets[(int64_t)tid * ntiles + blockIdx.x];
+  const int64_t tile = blockIdx.x;
+  // keys of the first round are loaded before the offsets are worked out
+  const int64_t tile0 = tile * kBlock * rounds;
+  K key = (tile0 + tid < num) ? kin[tile0 + tid] : (K)0;
+  {
+    uint32_t before = 0, total = 0;  // of digit tid: in the tiles before this one, in all tiles
+    if (FUSED) {
+      for (int64_t t0 = 0; t0 < ntiles; t0 += 8) {
+        uint32_t c[8];
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) wcnt[w][tid] = 0;
+        for (int j = 0; j < 8; ++j) c[j] = t0 + j < ntiles ? table[(t0 + j) * kBins + tid] : 0u;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          total += c[j];
+          if (t0 + j < tile) before += c[j];
+        }
+      }
+      if (clear) clear[tile * kBins + tid] = 0u;
+    } else {
+      before = table[(int64_t)tid * ntiles + tile];
+      total = totals[tid];
+    }
+    const int inc = wave_inclusive_sum((int)total);
+    if (lane == 63) wsum[wave] = (uint32_t)inc;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) wcnt[w][tid] = 0;
+    __syncthreads();
+    uint32_t lower = (uint32_t)inc - total;  // keys with a smaller digit
+    for (int w = 0; w < wave; ++w) lower += wsum[w];
+    base[tid] = lower + before;
+  }
   __syncthreads();
-  const int64_t tile0 = (int64_t)blockIdx.x * kBlock * rounds;
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  const int64_t tile_elems = (int64_t)kBlock * rounds;
   for (int r = 0; r < rounds; ++r) {
     const int64_t i = tile0 + (int64_t)r * kBlock + tid;
     const bool valid = i < num;
-    const K key = valid ? kin[i] : (K)0;
+    V val = V();
+    if (HAS_V && valid) val = vin[i];
+    K key_next = (K)0;
+    if (r + 1 < rounds && i + kBlock < num) key_next = kin[i + kBlock];
     const uint32_t d = (uint32_t)(key >> shift) & dmask;
     uint64_t peers = wave_ballot(valid);
 #pragma unroll
@@ -115,7 +171,11 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(const K *__restrict__ k
       uint32_t pos = base[d] + (uint32_t)rank;
       for (int w = 0; w < wave; ++w) pos += wcnt[w][d];
       kout[pos] = key;
-      if (HAS_V) vout[pos] = vin[i];
+      if (HAS_V) vout[pos] = val;
+      if (FUSED && next)
+        atomicAdd(&next[(int64_t)(pos / tile_elems) * kBins +
+                        ((uint32_t)(key >> next_shift) & next_dmask)],
+                  1u);
     }
     __syncthreads();
     {
@@ -128,6 +188,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(const K *__restrict__ k
       base[tid] += s;
     }
     __syncthreads();
+    key = key_next;
   }
 }
 
@@ -281,20 +342,48 @@ int sort_pairs(const K *kin, K *kout, const V *vin, V *vout, K *ktmp, V *vtmp, i
   const K *ksrc = kin;
   const V *vsrc = vin;
   bool to_out = (passes & 1) != 0;  // alternate so that the last pass writes kout/vout
+  uint32_t *totals = hist;
+  uint32_t *tables[3];
+  for (int i = 0; i < 3; ++i) tables[i] = hist + kBins + (p.fused ? i : 0) * (table_bytes(p) / 4);
+  const dim3 grid((unsigned)p.ntiles), block(kBlock);
+  auto digit_mask = [&](int shift) {
+    return end_bit - shift >= 8 ? 255u : ((1u << (end_bit - shift)) - 1u);
+  };
+  if (p.fused)
+    hist_kernel<K, true><<<grid, block, 0, st>>>(ksrc, num, begin_bit, digit_mask(begin_bit),
+                                                 p.rounds, p.ntiles, tables[0], tables[1]);
   for (int pass = 0; pass < passes; ++pass) {
     const int shift = begin_bit + 8 * pass;
-    const uint32_t dmask = end_bit - shift >= 8 ? 255u : ((1u << (end_bit - shift)) - 1u);
+    const uint32_t dmask = digit_mask(shift);
     K *kdst = to_out ? kout : ktmp;
     V *vdst = to_out ? vout : vtmp;
-    hist_kernel<K><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(ksrc, num, shift, dmask,
-                                                                     p.rounds, p.ntiles, hist);
-    hist_scan_kernel<<<dim3(1), dim3(kScanBlock), 0, st>>>(hist, p.ntiles * kBins);
-    if (has_v)
-      scatter_kernel<K, V, true><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(
-          ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, hist);
-    else
-      scatter_kernel<K, V, false><<<dim3((unsigned)p.ntiles), dim3(kBlock), 0, st>>>(
-          ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, hist);
+    if (p.fused) {
+      const bool last = pass + 1 == passes;
+      uint32_t *next = last ? nullptr : tables[(pass + 1) % 3];
+      uint32_t *clear = pass + 2 < passes ? tables[(pass + 2) % 3] : nullptr;
+      const int nshift = last ? 0 : shift + 8;
+      const uint32_t nmask = last ? 0u : digit_mask(nshift);
+      if (has_v)
+        scatter_kernel<K, V, true, true><<<grid, block, 0, st>>>(
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, tables[pass % 3],
+            nullptr, next, nshift, nmask, clear);
+      else
+        scatter_kernel<K, V, false, true><<<grid, block, 0, st>>>(
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, tables[pass % 3],
+            nullptr, next, nshift, nmask, clear);
+    } else {
+      hist_kernel<K, false><<<grid, block, 0, st>>>(ksrc, num, shift, dmask, p.rounds, p.ntiles,
+                                                    tables[0], nullptr);
+      digit_scan_kernel<<<dim3(kBins), block, 0, st>>>(tables[0], p.ntiles, totals);
+      if (has_v)
+        scatter_kernel<K, V, true, false><<<grid, block, 0, st>>>(
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, tables[0], totals,
+            nullptr, 0, 0u, nullptr);
+      else
+        scatter_kernel<K, V, false, false><<<grid, block, 0, st>>>(
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, tables[0], totals,
+            nullptr, 0, 0u, nullptr);
+    }
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     ksrc = kdst;
     vsrc = vdst;

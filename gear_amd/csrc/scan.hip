@@ -284,15 +284,31 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
     if (lane == kWave - 1) wtot[r][wave] = inc;
   }
   // sum of every earlier range (thread t takes ranges t, t+256, ...)
-  Acc part = (Acc)0;
-  for (int64_t j = tid; j < tile; j += kBlock) {
-    uint64_t v = load_agent(&aggr[j]);
-    while (v == kEmpty) {
-      __builtin_amdgcn_s_sleep(1);
-      v = load_agent(&aggr[j]);
-    }
-    part += Bits<Acc>::from(v);
+  // all of a thread's polls are issued together; only the ones not yet published are repeated
+  constexpr int kPolls = kMaxRanges / kBlock;
+  uint64_t pv[kPolls];
+#pragma unroll
+  for (int i = 0; i < kPolls; ++i) {
+    const int64_t j = tid + (int64_t)i * kBlock;
+    pv[i] = j < tile ? load_agent(&aggr[j]) : 0ull;
   }
+  bool pending = true;
+  while (pending) {
+    pending = false;
+#pragma unroll
+    for (int i = 0; i < kPolls; ++i) {
+      const int64_t j = tid + (int64_t)i * kBlock;
+      if (j < tile && pv[i] == kEmpty) {
+        pv[i] = load_agent(&aggr[j]);
+        pending |= pv[i] == kEmpty;
+      }
+    }
+    if (pending) __builtin_amdgcn_s_sleep(1);
+  }
+  Acc part = (Acc)0;
+#pragma unroll
+  for (int i = 0; i < kPolls; ++i)
+    if (tid + (int64_t)i * kBlock < tile) part += Bits<Acc>::from(pv[i]);
   const Acc pw = wave_sum(part);
   __syncthreads();  // wtot complete; everybody is done reading red
   if (lane == 0) red[wave] = pw;

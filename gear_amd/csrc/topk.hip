@@ -1,11 +1,11 @@
 // Top-k of fp32 priorities by radix select + ordered compaction + radix sort, gfx950.
 //
 // fp32 priorities map to order-preserving uint32 keys.  Three histogram passes (11 + 11 + 10
-// bits, LDS histograms, last finished workgroup picks the bin) find the key T of the k-th
-// largest priority and how many entries equal to T are still needed.  One compaction pass with a
-// decoupled look-back over packed (greater, equal) counts writes the selected entries in index
-// order: every entry above T, and the first need_eq entries equal to T -- ties go to the smaller
-// index.  For value order the k candidates then go through the stable LSD radix sort on the
+// bits, LDS histograms, the consuming launch picks the bin) find the key T of the k-th
+// largest priority and how many entries equal to T are still needed.  An ordered compaction (a
+// count launch and a write launch over packed (greater, equal) counts) writes the selected entries
+// in index order: every entry above T, and the first need_eq entries equal to T -- ties go to the
+// smaller index.  For value order the k candidates then go through the stable LSD radix sort on the
 // inverted key.
 #include "radix_sort.hpp"
 
@@ -13,16 +13,15 @@ namespace gearhip {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kRows = 4;
-constexpr int kTile = kBlock * kRows * 4;  // elements per compaction tile
+constexpr int kMaxRanges = 2048;  // workgroups of the compaction launches
+constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kHistBins = 2048;
 constexpr int kMaxHistBlocks = 512;
 
 struct State {
   uint32_t prefix[3];  // key bits decided after pass 0, 1, 2 (right-aligned)
   uint32_t k_rem[3];   // entries still to take from the bin picked in that pass
-  uint32_t ticket;     // tile ticket of the compaction pass
-  uint32_t pad[57];
+  uint32_t pad[58];
 };
 static_assert(sizeof(State) == 256, "State is the 256-byte header of the workspace");
 
@@ -38,11 +37,10 @@ struct Layout {
 
 Layout layout(int64_t n, int64_t k) {
   Layout l;
-  const int64_t tiles = n > 0 ? ceil_div64(n, kTile) : 0;
   const size_t kk = align_up((size_t)(k > 0 ? k : 1) * 4, 256);
   size_t o = sizeof(State);
   l.hist = o;  o += 3 * kHistBins * sizeof(uint32_t);
-  l.desc = o;  o += align_up((size_t)tiles * 8, 256);
+  l.desc = o;  o += (size_t)kMaxRanges * (kWavesPerBlock + 1) * 8;  // wave and workgroup counts
   l.ckey = o;  o += kk;
   l.cidx = o;  o += kk;
   l.skey = o;  o += kk;
@@ -149,246 +147,145 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__rest
     if (h[i]) atomicAdd(&hist[i], h[i]);
 }
 
-// packed per-tile descriptor: status (2 bits) | greater (31 bits) | equal (31 bits)
-constexpr uint64_t kStatusAggregate = 1ull << 62;
-constexpr uint64_t kStatusInclusive = 2ull << 62;
-constexpr uint64_t kCountMask = (1ull << 62) - 1;
+// Ordered compaction in two launches with no waiting between workgroups.  The input is cut into
+// gridDim.x * 4 contiguous wave ranges of wave_len elements (a multiple of kStep).  The count
+// launch writes every wave's packed (greater << 31 | equal) count and every workgroup's total; the
+// write launch sums the totals of the workgroups before it, adds the counts of the waves before it
+// in its own workgroup, and walks its range again (now from L2 / MALL) placing the selected entries.
+constexpr int kStep = kWave * 4;  // elements one wave handles per step (one float4 per lane)
+constexpr int kAhead = 4;         // steps whose loads are in flight together
 
-template <bool DIRECT>
-__global__ __launch_bounds__(kBlock) void compact_kernel(
-    const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist2,
-    uint64_t *desc,
-    uint32_t *__restrict__ ckey, uint32_t *__restrict__ cidx, float *__restrict__ values_out,
-    int64_t *__restrict__ indices_out) {
-  typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
-  constexpr int kWaves = kBlock / kWave;
-  __shared__ int wtot[kRows][kWaves];
-  __shared__ uint64_t s_excl;
-  __shared__ uint32_t s_tile;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid == 0) s_tile = atomicAdd(&state->ticket, 1u);
-  __syncthreads();
-  const int64_t tile = s_tile;
-  const int64_t base = tile * kTile;
-  const Pick pk = pick_bin<2>(k, state, hist2);
-  const uint32_t thr = pk.prefix;
-  const uint32_t need_eq = pk.k_rem;
+typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
 
-  uint32_t key[kRows][4];
-  int s[kRows];  // packed counts of the thread's vector: greater << 16 | equal
+__device__ __forceinline__ void load_quad(const float *__restrict__ p, int64_t e0, int64_t end,
+                                          float q[4]) {
+  if (e0 + 4 <= end) {
+    const f4 v = *reinterpret_cast<const f4 *>(p + e0);
+    q[0] = v[0]; q[1] = v[1]; q[2] = v[2]; q[3] = v[3];
+  } else {
 #pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * 4;
-    float q[4];
-    if (e0 + 4 <= n) {
-      const f4 v = *reinterpret_cast<const f4 *>(p + e0);
-      q[0] = v[0]; q[1] = v[1]; q[2] = v[2]; q[3] = v[3];
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) q[j] = (e0 + j < n) ? p[e0 + j] : 0.0f;
-    }
-    s[r] = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      key[r][j] = order_key(q[j]);
-      if (e0 + j < n) s[r] += key[r][j] > thr ? (1 << 16) : (key[r][j] == thr ? 1 : 0);
-    }
-  }
-  int wexcl[kRows];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int inc = wave_inclusive_sum(s[r]);
-    wexcl[r] = wave_shift_up1(inc);
-    if (lane == kWave - 1) wtot[r][wave] = inc;
-  }
-  __syncthreads();
-  int tile_total = 0;
-  int mybase[kRows];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    int acc = tile_total;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      if (w == wave) mybase[r] = acc + wexcl[r];
-      acc += wtot[r][w];
-    }
-    tile_total = acc;
-  }
-  const uint64_t tile_packed =
-      ((uint64_t)((uint32_t)tile_total >> 16) << 31) | (uint64_t)((uint32_t)tile_total & 0xffffu);
-
-  if (wave == 0) {
-    uint64_t excl = 0;
-    if (tile == 0) {
-      if (lane == 0) store_agent(&desc[0], kStatusInclusive | tile_packed);
-    } else {
-      if (lane == 0) store_agent(&desc[tile], kStatusAggregate | tile_packed);
-      int64_t look = tile - 1;
-      while (true) {
-        const int64_t idx = look - lane;
-        uint64_t v = kStatusInclusive;  // tiles before the first one: inclusive, zero counts
-        if (idx >= 0) v = load_agent(&desc[idx]);
-        const bool has_incl = (v >> 62) == 2;
-        const bool ready = (v >> 62) != 0;
-        const uint64_t bi = wave_ballot(has_incl), br = wave_ballot(ready);
-        const int first = bi ? (__ffsll((unsigned long long)bi) - 1) : kWave;
-        const uint64_t need = first >= 63 ? ~0ull : ((2ull << first) - 1ull);
-        if ((br & need) != need) {
-          __builtin_amdgcn_s_sleep(1);
-          continue;
-        }
-        const int64_t c = lane <= first ? (int64_t)(v & kCountMask) : 0;
-        excl += (uint64_t)wave_sum(c);
-        if (first < kWave) break;
-        look -= kWave;
-      }
-      if (lane == 0) store_agent(&desc[tile], kStatusInclusive | (excl + tile_packed));
-    }
-    if (lane == 0) s_excl = excl;
-  }
-  __syncthreads();
-  const uint32_t gt0 = (uint32_t)(s_excl >> 31);
-  const uint32_t eq0 = (uint32_t)(s_excl & 0x7fffffffu);
-
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * 4;
-    uint32_t gt = gt0 + ((uint32_t)mybase[r] >> 16);
-    uint32_t eq = eq0 + ((uint32_t)mybase[r] & 0xffffu);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      if (e0 + j < n) {
-        const bool is_gt = key[r][j] > thr, is_eq = key[r][j] == thr;
-        if (is_gt || (is_eq && eq < need_eq)) {
-          const uint32_t pos = gt + (eq < need_eq ? eq : need_eq);
-          if (DIRECT) {
-            indices_out[pos] = e0 + j;
-            if (values_out) values_out[pos] = p[e0 + j];
-          } else {
-            ckey[pos] = ~key[r][j];
-            cidx[pos] = (uint32_t)(e0 + j);
-          }
-        }
-        gt += is_gt;
-        eq += is_eq;
-      }
-    }
+    for (int j = 0; j < 4; ++j) q[j] = (e0 + j < end) ? p[e0 + j] : 0.0f;
   }
 }
 
-// Range variant of the compaction (cf. the range variant of the prefix sum): with at most
-// kMaxRanges workgroups every workgroup publishes its packed (greater, equal) count and takes the
-// sum of all earlier ranges' counts; no chain of inclusive values across the XCDs.
-constexpr int kMaxRanges = 2048;
-constexpr uint64_t kRangeReady = 1ull << 63;
-
-template <bool DIRECT, int NR>
-__global__ __launch_bounds__(kBlock) void compact_ranges_kernel(
+__global__ __launch_bounds__(kBlock) void count_ranges_kernel(
     const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist2,
-    uint64_t *desc,
+    int64_t wave_len, uint64_t *__restrict__ wave_counts, uint64_t *__restrict__ block_counts) {
+  __shared__ int64_t red[kWavesPerBlock];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t begin = gw * wave_len;
+  const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+  // the first loads are issued before the threshold is picked so that the two latencies overlap
+  float q[kAhead][4];
+#pragma unroll
+  for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
+  const uint32_t thr = pick_bin<2>(k, state, hist2).prefix;
+  uint32_t gt = 0, eq = 0;
+  for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
+    if (s0 != begin) {
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) load_quad(p, s0 + (int64_t)a * kStep + lane * 4, end, q[a]);
+    }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) {
+      const int64_t e0 = s0 + (int64_t)a * kStep + lane * 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t key = order_key(q[a][j]);
+        if (e0 + j < end) {
+          gt += key > thr;
+          eq += key == thr;
+        }
+      }
+    }
+  }
+  const int64_t w = wave_sum(((int64_t)gt << 31) | (int64_t)eq);
+  if (lane == 0) {
+    wave_counts[gw] = (uint64_t)w;
+    red[wave] = w;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int64_t t = 0;
+#pragma unroll
+    for (int i = 0; i < kWavesPerBlock; ++i) t += red[i];
+    block_counts[blockIdx.x] = (uint64_t)t;
+  }
+}
+
+template <bool DIRECT>
+__global__ __launch_bounds__(kBlock) void write_ranges_kernel(
+    const float *__restrict__ p, int64_t n, const State *state, int64_t wave_len,
+    const uint64_t *__restrict__ wave_counts, const uint64_t *__restrict__ block_counts,
     uint32_t *__restrict__ ckey, uint32_t *__restrict__ cidx, float *__restrict__ values_out,
     int64_t *__restrict__ indices_out) {
-  typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
-  constexpr int kWaves = kBlock / kWave;
-  constexpr int kElems = NR * kBlock * 4;
-  __shared__ int wtot[NR][kWaves];
-  __shared__ int64_t red[kWaves];
-  __shared__ uint32_t s_tile;
+  __shared__ int64_t red[kWavesPerBlock];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid == 0) s_tile = atomicAdd(&state->ticket, 1u);
-  __syncthreads();
-  const int64_t tile = s_tile;
-  const int64_t base = tile * kElems;
-  const Pick pk = pick_bin<2>(k, state, hist2);
-  const uint32_t thr = pk.prefix;
-  const uint32_t need_eq = pk.k_rem;
+  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t begin = gw * wave_len;
+  const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+  float q[kAhead][4];
+#pragma unroll
+  for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
+  const uint32_t thr = state->prefix[2];
+  const uint32_t need_eq = state->k_rem[2];
 
-  float q[NR][4];
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * 4;
-    if (e0 + 4 <= n) {
-      const f4 v = *reinterpret_cast<const f4 *>(p + e0);
-      q[r][0] = v[0]; q[r][1] = v[1]; q[r][2] = v[2]; q[r][3] = v[3];
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) q[r][j] = (e0 + j < n) ? p[e0 + j] : 0.0f;
-    }
-  }
-  int s[NR];  // packed counts of the thread's vector: greater << 16 | equal
-  int64_t tsum = 0;  // greater << 31 | equal over the thread's vectors
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * 4;
-    s[r] = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t key = order_key(q[r][j]);
-      if (e0 + j < n) s[r] += key > thr ? (1 << 16) : (key == thr ? 1 : 0);
-    }
-    tsum += ((int64_t)(s[r] >> 16) << 31) | (int64_t)(s[r] & 0xffff);
-  }
-  {
-    const int64_t w = wave_sum(tsum);
-    if (lane == 0) red[wave] = w;
-    __syncthreads();
-    if (tid == 0)
-      store_agent(&desc[tile], kRangeReady | (uint64_t)(red[0] + red[1] + red[2] + red[3]));
-  }
-  int wexcl[NR];
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    const int inc = wave_inclusive_sum(s[r]);
-    wexcl[r] = wave_shift_up1(inc);
-    if (lane == kWave - 1) wtot[r][wave] = inc;
-  }
   int64_t part = 0;
-  for (int64_t j = tid; j < tile; j += kBlock) {
-    uint64_t v = load_agent(&desc[j]);
-    while (!(v & kRangeReady)) {
-      __builtin_amdgcn_s_sleep(1);
-      v = load_agent(&desc[j]);
-    }
-    part += (int64_t)(v & ~kRangeReady);
-  }
+  for (int j = tid; j < (int)blockIdx.x; j += kBlock) part += (int64_t)block_counts[j];
   const int64_t pw = wave_sum(part);
-  __syncthreads();
   if (lane == 0) red[wave] = pw;
   __syncthreads();
-  const int64_t excl = red[0] + red[1] + red[2] + red[3];
-  uint32_t gt_row = (uint32_t)(excl >> 31), eq_row = (uint32_t)(excl & 0x7fffffff);
+  int64_t excl = 0;
+#pragma unroll
+  for (int i = 0; i < kWavesPerBlock; ++i) excl += red[i];
+  // plus the waves before this one in its own workgroup
+  int64_t own = 0;
+  if (lane < wave) own = (int64_t)wave_counts[(int64_t)blockIdx.x * kWavesPerBlock + lane];
+  excl += wave_sum(own);
+  uint32_t gt_run = (uint32_t)(excl >> 31), eq_run = (uint32_t)(excl & 0x7fffffff);
 
+  for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
+    if (s0 != begin) {
 #pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    int before = 0, mine = 0;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      if (w == wave) mine = before + wexcl[r];
-      before += wtot[r][w];
+      for (int a = 0; a < kAhead; ++a) load_quad(p, s0 + (int64_t)a * kStep + lane * 4, end, q[a]);
     }
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * 4;
-    uint32_t gt = gt_row + ((uint32_t)mine >> 16);
-    uint32_t eq = eq_row + ((uint32_t)mine & 0xffffu);
-    gt_row += (uint32_t)before >> 16;
-    eq_row += (uint32_t)before & 0xffffu;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      if (e0 + j < n) {
-        const uint32_t key = order_key(q[r][j]);
-        const bool is_gt = key > thr, is_eq = key == thr;
-        if (is_gt || (is_eq && eq < need_eq)) {
-          const uint32_t pos = gt + (eq < need_eq ? eq : need_eq);
-          if (DIRECT) {
-            indices_out[pos] = e0 + j;
-            if (values_out) values_out[pos] = q[r][j];
-          } else {
-            ckey[pos] = ~key;
-            cidx[pos] = (uint32_t)(e0 + j);
-          }
-        }
-        gt += is_gt;
-        eq += is_eq;
+    for (int a = 0; a < kAhead; ++a) {
+      const int64_t e0 = s0 + (int64_t)a * kStep + lane * 4;
+      uint32_t key[4];
+      int s = 0;  // packed counts of the lane's four entries: greater << 16 | equal
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        key[j] = order_key(q[a][j]);
+        if (e0 + j < end) s += key[j] > thr ? (1 << 16) : (key[j] == thr ? 1 : 0);
       }
+      if (wave_ballot(s != 0) == 0ull) continue;
+      const int inc = wave_inclusive_sum(s);
+      const int total = wave_read_lane(inc, kWave - 1);
+      const int before = inc - s;
+      uint32_t g = gt_run + ((uint32_t)before >> 16);
+      uint32_t e = eq_run + ((uint32_t)before & 0xffffu);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (e0 + j < end) {
+          const bool is_gt = key[j] > thr, is_eq = key[j] == thr;
+          if (is_gt || (is_eq && e < need_eq)) {
+            const uint32_t pos = g + (e < need_eq ? e : need_eq);
+            if (DIRECT) {
+              indices_out[pos] = e0 + j;
+              if (values_out) values_out[pos] = q[a][j];
+            } else {
+              ckey[pos] = ~key[j];
+              cidx[pos] = (uint32_t)(e0 + j);
+            }
+          }
+          g += is_gt;
+          e += is_eq;
+        }
+      }
+      gt_run += (uint32_t)total >> 16;
+      eq_run += (uint32_t)total & 0xffffu;
     }
   }
 }
@@ -428,7 +325,7 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   uint64_t *desc = reinterpret_cast<uint64_t *>(ws + l.desc);
   hipStream_t st = as_stream(stream);
 
-  const int64_t zero_words = (int64_t)(l.ckey / 4);  // header + histograms + descriptors
+  const int64_t zero_words = (int64_t)(l.desc / 4);  // header + histograms
   zero_kernel<<<dim3((unsigned)ceil_div64(zero_words, 256)), dim3(256), 0, st>>>(
       reinterpret_cast<uint32_t *>(ws), zero_words);
   int64_t hblocks = ceil_div64(n, (int64_t)kBlock * 4 * 4);
@@ -443,36 +340,23 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   uint32_t *ckey = reinterpret_cast<uint32_t *>(ws + l.ckey);
   uint32_t *cidx = reinterpret_cast<uint32_t *>(ws + l.cidx);
   const bool direct = !sorted_by_value;
-  const int64_t row = (int64_t)kBlock * 4;
-#define GEARHIP_COMPACT_RANGES(NR)                                                              \
-  do {                                                                                          \
-    const unsigned g = (unsigned)ceil_div64(n, (NR) * row);                                     \
-    if (direct)                                                                                 \
-      compact_ranges_kernel<true, NR><<<dim3(g), block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins, desc,    \
-                                                                 ckey, cidx, values_out,        \
-                                                                 indices_out);                  \
-    else                                                                                        \
-      compact_ranges_kernel<false, NR><<<dim3(g), block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins, desc,   \
-                                                                  ckey, cidx, values_out,       \
-                                                                  indices_out);                 \
-  } while (0)
-  if (ceil_div64(n, 4 * row) <= 1024) {
-    GEARHIP_COMPACT_RANGES(4);
-  } else if (ceil_div64(n, 8 * row) <= 1024) {
-    GEARHIP_COMPACT_RANGES(8);
-  } else if (ceil_div64(n, 16 * row) <= kMaxRanges) {
-    GEARHIP_COMPACT_RANGES(16);
-  } else {
-    const int64_t tiles = ceil_div64(n, kTile);
-    if (direct)
-      compact_kernel<true><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins, desc, ckey,
-                                                                    cidx, values_out, indices_out);
-    else
-      compact_kernel<false><<<dim3((unsigned)tiles), block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins, desc,
-                                                                     ckey, cidx, values_out,
-                                                                     indices_out);
-  }
-#undef GEARHIP_COMPACT_RANGES
+  int64_t ranges = ceil_div64(n, (int64_t)kWavesPerBlock * kAhead * kStep);
+  if (ranges > kMaxRanges) ranges = kMaxRanges;
+  const int64_t wave_len = ceil_div64(ceil_div64(n, ranges * kWavesPerBlock), kStep) * kStep;
+  ranges = ceil_div64(n, wave_len * kWavesPerBlock);
+  uint64_t *wave_counts = reinterpret_cast<uint64_t *>(ws + l.desc);
+  uint64_t *block_counts = wave_counts + (size_t)kMaxRanges * kWavesPerBlock;
+  const dim3 cgrid((unsigned)ranges);
+  count_ranges_kernel<<<cgrid, block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins,
+                                               wave_len, wave_counts, block_counts);
+  if (direct)
+    write_ranges_kernel<true><<<cgrid, block, 0, st>>>(priorities, n, state, wave_len, wave_counts,
+                                                       block_counts, ckey, cidx, values_out,
+                                                       indices_out);
+  else
+    write_ranges_kernel<false><<<cgrid, block, 0, st>>>(priorities, n, state, wave_len,
+                                                        wave_counts, block_counts, ckey, cidx,
+                                                        values_out, indices_out);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   if (direct) return 0;
   uint32_t *skey = reinterpret_cast<uint32_t *>(ws + l.skey);
