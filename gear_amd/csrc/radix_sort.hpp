@@ -114,6 +114,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   __shared__ uint32_t base[kBins];
   __shared__ uint32_t wcnt[kWaves][kBins];
   __shared__ uint32_t wsum[kWaves];
+  __shared__ uint32_t part[FUSED ? kWaves : 1][2][kBins];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t tile = blockIdx.x;
   // keys of the first round are loaded before the offsets are worked out
@@ -122,15 +123,37 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   {
     uint32_t before = 0, total = 0;  // of digit tid: in the tiles before this one, in all tiles
     if (FUSED) {
-      for (int64_t t0 = 0; t0 < ntiles; t0 += 8) {
-        uint32_t c[8];
+      // lane q of wave g sums digits 4q..4q+3 over the tiles g, g + 4, g + 8, ...: sixteen
+      // 16-byte loads in flight per lane; the four waves' parts meet in LDS
+      uint32_t bef[4] = {0u, 0u, 0u, 0u}, tot[4] = {0u, 0u, 0u, 0u};
+      for (int64_t t0 = wave; t0 < ntiles; t0 += kWaves * 16) {
+        u32x4 c[16];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) c[j] = t0 + j < ntiles ? table[(t0 + j) * kBins + tid] : 0u;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          total += c[j];
-          if (t0 + j < tile) before += c[j];
+        for (int j = 0; j < 16; ++j) {
+          const int64_t t = t0 + (int64_t)j * kWaves;
+          c[j] = u32x4{0u, 0u, 0u, 0u};
+          if (t < ntiles) c[j] = *reinterpret_cast<const u32x4 *>(table + t * kBins + 4 * lane);
         }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const bool earlier = t0 + (int64_t)j * kWaves < tile;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            tot[i] += c[j][i];
+            if (earlier) bef[i] += c[j][i];
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        part[wave][0][4 * lane + i] = bef[i];
+        part[wave][1][4 * lane + i] = tot[i];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        before += part[w][0][tid];
+        total += part[w][1][tid];
       }
       if (clear) clear[tile * kBins + tid] = 0u;
     } else {

@@ -134,12 +134,25 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__rest
     }
   };
   const int64_t nvec = n >> 2;
-  for (int64_t v = (int64_t)blockIdx.x * kBlock + tid; v < nvec; v += (int64_t)gridDim.x * kBlock) {
-    const f4 q = *reinterpret_cast<const f4 *>(p + (v << 2));
-    count(q[0]);
-    count(q[1]);
-    count(q[2]);
-    count(q[3]);
+  constexpr int kLoads = 4;  // 16-byte loads in flight per thread
+  for (int64_t v0 = (int64_t)blockIdx.x * kBlock * kLoads + tid; v0 < nvec;
+       v0 += (int64_t)gridDim.x * kBlock * kLoads) {
+    f4 q[kLoads];
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int64_t v = v0 + (int64_t)u * kBlock;
+      q[u] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (v < nvec) q[u] = *reinterpret_cast<const f4 *>(p + (v << 2));
+    }
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      if (v0 + (int64_t)u * kBlock < nvec) {
+        count(q[u][0]);
+        count(q[u][1]);
+        count(q[u][2]);
+        count(q[u][3]);
+      }
+    }
   }
   if (blockIdx.x == 0 && tid < (int)(n & 3)) count(p[(nvec << 2) + tid]);
   __syncthreads();

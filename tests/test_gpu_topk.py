@@ -61,7 +61,8 @@ def test_sort_i64(oracle):
     from gear_amd import ops
     rng = np.random.default_rng(41)
     for n, bits in ((1, 1), (2, 8), (255, 9), (256, 20), (1025, 20), (2048, 24), (4096, 31),
-                    (65_536, 40), (300_001, 63)):
+                    (4097, 17), (5000, 64), (65_536, 40), (131_072, 33), (131_073, 16),
+                    (300_001, 63)):
         keys = rng.integers(0, 1 << min(bits, 62), size=n).astype(np.int64)
         keys[rng.integers(0, n, size=max(n // 3, 1))] = keys[0]  # duplicates: stability matters
         vals = rng.integers(-2**62, 2**62, size=n).astype(np.int64)
