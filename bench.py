@@ -199,9 +199,8 @@ def cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst):
     T = tab.T
     rng = np.random.default_rng(3004)
     dsts = [np.zeros((B, span * sb), np.uint8) for sb in tab.step_bytes]
-    nrun, t_total = 0, 0.0
-    budget = 12.0
-    while nrun < 3 or (t_total < budget and nrun < 20):
+
+    def one_step(threads):
         u01 = rng.random(B, dtype=np.float32)
         t0 = time.perf_counter()
         prefix = orc.scan_f32_f64(pri)
@@ -212,17 +211,46 @@ def cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst):
         lens = tss + 1
         for c in range(4):
             orc.subcopy(host, idxs, tss, lens, True, ofst, span, tab.traj_stride,
-                        tab.step_bytes[c], tab.col_base(c), zero_fill=True, dst=dsts[c])
-        t_total += time.perf_counter() - t0
-        nrun += 1
+                        tab.step_bytes[c], tab.col_base(c), zero_fill=True, dst=dsts[c],
+                        threads=threads)
+        return time.perf_counter() - t0
+
+    def timed(threads, budget):
+        nrun, t_total = 0, 0.0
+        while nrun < 3 or (t_total < budget and nrun < 400):
+            t_total += one_step(threads)
+            nrun += 1
+        return nrun, t_total
+
+    nrun, t_total = timed(1, 10.0)
+    # the gather over the host's share of cores (windows split over threads; scan, search and sort
+    # stay sequential): 16 threads at most, the CPU share of a one-GPU box
+    cores = max(1, min(16, os.cpu_count() or 1))
+    one_step(cores)
+    nrun_mt, t_mt = timed(cores, 5.0)
     return {"value": B * nrun / t_total, "unit": "windows/s", "cores": 1, "kind": "port",
             "ms_per_step": t_total / nrun * 1e3,
+            "all_cores": {"value": B * nrun_mt / t_mt, "unit": "windows/s", "cores": cores,
+                          "ms_per_step": t_mt / nrun_mt * 1e3},
+            "cpu_model": cpu_model(),
             "sample": "%d steps of the same pipeline (fp64 scan of 1e6 priorities, 2048 searches, "
                       "sort, 4-column gather with memset+memcpy per window) on the first %d of %d "
                       "trajectories (%.1f GB of the table, trajectory index taken modulo %d); "
-                      "host has %d logical cores, 1 used"
+                      "host has %d logical cores; value uses 1, all_cores splits the gather's "
+                      "windows over %d threads (%d steps)"
                       % (nrun, keep, tab.capacity, keep * tab.traj_stride / 1e9, keep,
-                         os.cpu_count() or 0)}
+                         os.cpu_count() or 0, cores, nrun_mt)}
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 class GenericTable:

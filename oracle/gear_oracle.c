@@ -10,6 +10,7 @@
  *   oracle_layout        closed form + tests/test_table.py:15-24 sizes            (pinned)
  *   oracle_sub           hand vector from tests/test_sub.py:10-28 + brute force   (pinned)
  *   oracle_subcopy       numpy fancy-index gather + examples/.../misc.py:16-29    (pinned)
+ *   oracle_subcopy_mt    equality with oracle_subcopy                             (pinned)
  *   oracle_vcopy/copy    numpy slicing + tests/test_copy.py:5-28                  (pinned)
  *   oracle_scan_*        numpy.cumsum (fp64 / int64), integer-valued closed forms (pinned)
  *   oracle_sum_f32       math.fsum                                                (pinned)
@@ -117,6 +118,25 @@ ORACLE_API void oracle_subcopy(const uint8_t *src, uint8_t *dst, int64_t num,
       for (int64_t j = 0; j < span; ++j)
         mask[g * span + j] = pad_head ? (uint8_t)(j >= span - steps) : (uint8_t)(j < steps);
     }
+  }
+}
+
+/* The same gather with the windows split over `threads` host threads (windows are independent
+ * units; each thread runs oracle_subcopy on a contiguous share).  Only the all-cores leg of the
+ * CPU baseline uses it; results are identical to oracle_subcopy by construction (tested).    */
+ORACLE_API void oracle_subcopy_mt(const uint8_t *src, uint8_t *dst, int64_t num,
+                                  const int64_t *idxs, const int64_t *tss, const int64_t *lens,
+                                  int pad_head, int64_t ofst, int64_t span, int64_t traj_stride,
+                                  int64_t step_bytes, int64_t col_base, int64_t dst_stride,
+                                  int zero_fill, uint8_t *mask, int threads) {
+  if (threads < 1) threads = 1;
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int t = 0; t < threads; ++t) {
+    const int64_t lo = num * t / threads, hi = num * (t + 1) / threads;
+    if (hi > lo)
+      oracle_subcopy(src, dst + dst_stride * lo, hi - lo, idxs + lo, tss + lo, lens + lo, pad_head,
+                     ofst, span, traj_stride, step_bytes, col_base, dst_stride, zero_fill,
+                     mask ? mask + lo * span : NULL);
   }
 }
 

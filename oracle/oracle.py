@@ -67,8 +67,9 @@ def sub(idxs, tss, lens, pad_head, ofst, span, traj_stride, step_bytes, col_base
 
 
 def subcopy(table, idxs, tss, lens, pad_head, ofst, span, traj_stride, step_bytes, col_base,
-            dst_stride=None, zero_fill=True, want_mask=False, dst=None):
-    """Returns (dst uint8[num, dst_stride], mask uint8[num, span] or None)."""
+            dst_stride=None, zero_fill=True, want_mask=False, dst=None, threads=1):
+    """Returns (dst uint8[num, dst_stride], mask uint8[num, span] or None).  threads > 1 splits
+    the windows over that many host threads (same result)."""
     table = _c(table, np.uint8)
     idxs, tss, lens = _c(idxs, np.int64), _c(tss, np.int64), _c(lens, np.int64)
     n = len(idxs)
@@ -77,13 +78,17 @@ def subcopy(table, idxs, tss, lens, pad_head, ofst, span, traj_stride, step_byte
     if dst is None:
         dst = np.zeros((n, dst_stride), np.uint8)
     mask = np.zeros((n, span), np.uint8) if want_mask else None
-    lib().oracle_subcopy(_p(table, _u8p), _p(dst, _u8p), ctypes.c_int64(n), _p(idxs, _i64p),
-                         _p(tss, _i64p), _p(lens, _i64p), ctypes.c_int(int(pad_head)),
-                         ctypes.c_int64(ofst), ctypes.c_int64(span),
-                         ctypes.c_int64(traj_stride), ctypes.c_int64(step_bytes),
-                         ctypes.c_int64(col_base), ctypes.c_int64(dst_stride),
-                         ctypes.c_int(int(zero_fill)),
-                         _p(mask, _u8p) if want_mask else None)
+    args = [_p(table, _u8p), _p(dst, _u8p), ctypes.c_int64(n), _p(idxs, _i64p),
+            _p(tss, _i64p), _p(lens, _i64p), ctypes.c_int(int(pad_head)),
+            ctypes.c_int64(ofst), ctypes.c_int64(span),
+            ctypes.c_int64(traj_stride), ctypes.c_int64(step_bytes),
+            ctypes.c_int64(col_base), ctypes.c_int64(dst_stride),
+            ctypes.c_int(int(zero_fill)),
+            _p(mask, _u8p) if want_mask else None]
+    if threads > 1:
+        lib().oracle_subcopy_mt(*args, ctypes.c_int(int(threads)))
+    else:
+        lib().oracle_subcopy(*args)
     return dst, mask
 
 

@@ -159,3 +159,21 @@ def test_zero_fill_flag(oracle):
     keep = np.repeat(mask, 3, axis=1).astype(bool)
     assert np.array_equal(dst[keep], ref[keep])
     assert np.all(dst[~keep] == 0xEE)
+
+
+def test_subcopy_threads_equal_single_thread(oracle):
+    """The all-cores leg of the CPU baseline splits the windows over threads: same bytes, same mask."""
+    rng = np.random.default_rng(77)
+    T, cap, sb = 16, 9, 7
+    stride = T * (sb + 3)
+    table = rng.integers(0, 256, size=cap * stride, dtype=np.uint8)
+    n = 37
+    idxs = rng.integers(0, cap, size=n).astype(np.int64)
+    lens = rng.integers(0, T + 1, size=n).astype(np.int64)
+    tss = rng.integers(0, T, size=n).astype(np.int64)
+    for pad_head in (False, True):
+        a, ma = oracle.subcopy(table, idxs, tss, lens, pad_head, -3, 6, stride, sb, 0, want_mask=True)
+        for threads in (2, 5, 64):
+            b, mb = oracle.subcopy(table, idxs, tss, lens, pad_head, -3, 6, stride, sb, 0,
+                                   want_mask=True, threads=threads)
+            assert np.array_equal(a, b) and np.array_equal(ma, mb)
