@@ -1,15 +1,21 @@
-// Single-pass inclusive prefix sum (decoupled look-back) and a deterministic sum, gfx950.
+// Inclusive prefix sums and a deterministic sum, gfx950.  fp32 inputs are accumulated in fp64.
 //
-// A tile is 256 threads x 4 rows of 16-byte input vectors, read with the lanes of a wave on
-// consecutive vectors (coalesced).  Each thread scans inside its vectors, the four row sums go
-// through a DPP wave scan, wave totals meet in LDS, and the tile's exclusive prefix comes from the
-// tiles before it through two 64-bit words per tile in the workspace:
-//     aggr[t]  sum of tile t alone            incl[t]  sum of tiles 0..t
-// A word equal to kEmpty means "not published yet"; value and readiness travel in one agent-scope
-// 64-bit store, so no fence pairs are needed.  Tile numbers are handed out by an atomic ticket in
-// launch order, hence every predecessor a tile waits for is already running.
-// Wave 0 of a tile looks back 64 predecessors at a time (one per lane, ballots pick the nearest
-// published inclusive value).  fp32 inputs are accumulated in fp64.
+// Three kernels share the inner scan (each thread scans inside its 16-byte input vectors, row sums
+// go through a DPP wave scan, wave totals meet in LDS, results leave through LDS so that every store
+// instruction writes whole lines):
+//  * default, up to 2048 ranges (n <= 33.5 M fp32): two launches.  range_sum_kernel writes the sum
+//    of every range; scan_ranges_kernel<TWO = true> re-reads its range (now in L2 / MALL), adds
+//    the sums of all earlier ranges in a fixed order and writes the prefix.  No workgroup waits for
+//    another one.  On this multi-XCD part that is faster than the one-pass kernels: a ticket per
+//    workgroup on one address costs ~19 ns each across the XCDs, and every agent-scope round trip
+//    of a look-back 1-2 us.
+//  * GEAR_HIP_SCAN_SINGLE_PASS=1: scan_ranges_kernel<TWO = false>, one pass over the data.  Tile
+//    numbers are handed out by an atomic ticket in launch order (every awaited predecessor is
+//    already running); a workgroup publishes the sum of its range in one agent-scope 64-bit store
+//    (kEmpty = not published, so no fence pairs) and sums ALL earlier ranges' words.
+//  * beyond 2048 ranges: scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone,
+//    incl[t] = sum of tiles 0..t; wave 0 looks back 64 predecessors at a time, ballots pick the
+//    nearest published inclusive value).
 #include "wave.hpp"
 
 namespace gearhip {
@@ -228,7 +234,45 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
 // is no serial chain across the XCDs, and the result is bit-reproducible from run to run.
 constexpr int kMaxRanges = 2048;
 
-template <typename In, typename Acc, typename Out, int VE, int NR>
+// Sum of every range, one workgroup per range: the first launch of the two-launch variant, in
+// which the scan launch below finds all aggregates ready (no ticket, no publishing, no polling).
+template <typename In, typename Acc, int VE, int NR>
+__global__ __launch_bounds__(kBlock) void range_sum_kernel(const In *__restrict__ in, int64_t n,
+                                                           uint64_t *__restrict__ aggr) {
+  constexpr int kElems = NR * kBlock * VE;
+  constexpr int kWaves = kBlock / kWave;
+  typedef typename InVec<In, VE>::type in_vec;
+  __shared__ Acc red[kWaves];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  const int64_t base = (int64_t)blockIdx.x * kElems;
+  In raw[NR][VE];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
+    if (e0 + VE <= n) {
+      const in_vec v = *reinterpret_cast<const in_vec *>(in + e0);
+#pragma unroll
+      for (int j = 0; j < VE; ++j) raw[r][j] = v[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < VE; ++j) raw[r][j] = (e0 + j < n) ? in[e0 + j] : (In)0;
+    }
+  }
+  Acc tsum = (Acc)0;
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    Acc a = (Acc)raw[r][0];
+#pragma unroll
+    for (int j = 1; j < VE; ++j) a += (Acc)raw[r][j];
+    tsum += a;
+  }
+  const Acc w = wave_sum(tsum);
+  if (lane == 0) red[wave] = w;
+  __syncthreads();
+  if (tid == 0) aggr[blockIdx.x] = Bits<Acc>::to((red[0] + red[1]) + (red[2] + red[3]));
+}
+
+template <typename In, typename Acc, typename Out, int VE, int NR, bool TWO>
 __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restrict__ in,
                                                              Out *__restrict__ out, int64_t n,
                                                              uint32_t *ticket, uint64_t *aggr) {
@@ -241,9 +285,11 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
   __shared__ uint32_t s_tile;
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-  if (tid == 0) s_tile = atomicAdd(ticket, 1u);
-  __syncthreads();
-  const int64_t tile = s_tile;
+  if (!TWO) {
+    if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+    __syncthreads();
+  }
+  const int64_t tile = TWO ? (int64_t)blockIdx.x : (int64_t)s_tile;
   const int64_t base = tile * kElems;
 
   In raw[NR][VE];
@@ -270,7 +316,7 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
     tsum += a;
   }
   // the range's aggregate goes out before the detailed scan
-  {
+  if (!TWO) {
     const Acc w = wave_sum(tsum);
     if (lane == 0) red[wave] = w;
     __syncthreads();
@@ -290,9 +336,9 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
 #pragma unroll
   for (int i = 0; i < kPolls; ++i) {
     const int64_t j = tid + (int64_t)i * kBlock;
-    pv[i] = j < tile ? load_agent(&aggr[j]) : 0ull;
+    pv[i] = j < tile ? (TWO ? aggr[j] : load_agent(&aggr[j])) : 0ull;
   }
-  bool pending = true;
+  bool pending = !TWO;
   while (pending) {
     pending = false;
 #pragma unroll
@@ -383,14 +429,21 @@ size_t scan_ws_bytes(int64_t n) {
 }
 
 template <typename In, typename Acc, typename Out, int VE, int NR>
-int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st) {
+int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, bool single_pass) {
   const int64_t ranges = ceil_div64(n, (int64_t)NR * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
   uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
+  if (!single_pass) {
+    range_sum_kernel<In, Acc, VE, NR><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(in, n, aggr);
+    scan_ranges_kernel<In, Acc, Out, VE, NR, true><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(
+        in, out, n, ticket, aggr);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
   scan_init_kernel<<<dim3((unsigned)ceil_div64(ranges, kBlock)), dim3(kBlock), 0, st>>>(ticket, aggr,
                                                                                       ranges);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  scan_ranges_kernel<In, Acc, Out, VE, NR><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(
+  scan_ranges_kernel<In, Acc, Out, VE, NR, false><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(
       in, out, n, ticket, aggr);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -406,12 +459,21 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
   if ((reinterpret_cast<uintptr_t>(in) & (sizeof(In) - 1)) ||
       (reinterpret_cast<uintptr_t>(out) & 15))
     return GEAR_HIP_EALIGN;
-  // few enough ranges: no look-back chain (4, 8 or 16 rows of 256 vectors per workgroup)
   const int64_t row = (int64_t)kBlock * VE;
-  if (ceil_div64(n, 4 * row) <= 1024) return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st);
-  if (ceil_div64(n, 8 * row) <= 1024) return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st);
+  // Up to 2048 ranges of 2, 4, 8 or 16 rows of 256 vectors.  Default: two launches (range sums,
+  // then the scan with every aggregate ready).  GEAR_HIP_SCAN_SINGLE_PASS=1 selects the one-pass
+  // kernel with tickets and published aggregates instead (larger ranges, so that all workgroups
+  // are resident together).
+  const bool single_pass = env_int("GEAR_HIP_SCAN_SINGLE_PASS", 0) != 0;
+  const int64_t cap = single_pass ? 1024 : kMaxRanges;
+  if (!single_pass && ceil_div64(n, 2 * row) <= cap)
+    return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, single_pass);
+  if (ceil_div64(n, 4 * row) <= cap)
+    return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, single_pass);
+  if (ceil_div64(n, 8 * row) <= cap)
+    return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, single_pass);
   if (ceil_div64(n, 16 * row) <= kMaxRanges)
-    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st);
+    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, single_pass);
   const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
   uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);

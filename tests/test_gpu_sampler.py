@@ -1,5 +1,8 @@
-"""GPU parity of the weighted sampler: fp64 prefix sum (decoupled look-back scan), batched
-upper_bound search, importance weights, through the C ABI against the CPU oracle."""
+"""GPU parity of the weighted sampler: fp64 prefix sum (both variants of the range scan and the
+tiled look-back scan for very long inputs), batched upper_bound search, importance weights, through
+the C ABI against the CPU oracle."""
+import os
+
 import numpy as np
 import pytest
 
@@ -8,8 +11,20 @@ from conftest import announce
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
 
-SIZES = [1, 2, 3, 63, 64, 65, 255, 1023, 4095, 4096, 4097, 8191, 8192, 8193, 100_000,
-         1_000_000, 10_000_003]
+SIZES = [1, 2, 3, 63, 64, 65, 255, 1023, 2047, 2048, 2049, 4095, 4096, 4097, 8191, 8192, 8193,
+         100_000, 1_000_000, 4_194_305, 10_000_003, 34_000_001]
+
+
+@pytest.fixture(params=["two_launch", "single_pass"])
+def scan_variant(request):
+    """The library reads GEAR_HIP_SCAN_SINGLE_PASS at every call."""
+    old = os.environ.get("GEAR_HIP_SCAN_SINGLE_PASS")
+    os.environ["GEAR_HIP_SCAN_SINGLE_PASS"] = "1" if request.param == "single_pass" else "0"
+    yield request.param
+    if old is None:
+        os.environ.pop("GEAR_HIP_SCAN_SINGLE_PASS", None)
+    else:
+        os.environ["GEAR_HIP_SCAN_SINGLE_PASS"] = old
 
 
 def _dev(a):
@@ -22,13 +37,13 @@ def _priorities(n, seed):
 
 
 @pytest.mark.parametrize("n", SIZES)
-def test_scan_integer_valued_is_bit_exact(oracle, n):
+def test_scan_integer_valued_is_bit_exact(oracle, n, scan_variant):
     """Integer-valued fp32 priorities: every partial sum is exact in fp64, so any summation order
     must reproduce the sequential oracle bit for bit."""
     from gear_amd import ops
     rng = np.random.default_rng(n)
     p = rng.integers(0, 1000, size=n).astype(np.float32)
-    announce("scan integer-valued n=%d" % n)
+    announce("scan integer-valued n=%d %s" % (n, scan_variant))
     got = ops.prefix_sum(_dev(p))
     torch.cuda.synchronize()
     exp = oracle.scan_f32_f64(p)
@@ -37,12 +52,12 @@ def test_scan_integer_valued_is_bit_exact(oracle, n):
 
 
 @pytest.mark.parametrize("n", [1, 4097, 1_000_000, 10_000_003])
-def test_scan_lognormal_close_to_sequential(oracle, n):
+def test_scan_lognormal_close_to_sequential(oracle, n, scan_variant):
     """Random priorities: the parallel fp64 sum may differ from the sequential one in the last
     bits only: relative error <= 1e-12 (tolerance of the fp64 prefix), and it is monotone."""
     from gear_amd import ops
     p = _priorities(n, 1002)
-    announce("scan lognormal n=%d" % n)
+    announce("scan lognormal n=%d %s" % (n, scan_variant))
     got = ops.prefix_sum(_dev(p)).cpu().numpy()
     exp = oracle.scan_f32_f64(p)
     rel = np.max(np.abs(got - exp) / exp)
@@ -50,9 +65,10 @@ def test_scan_lognormal_close_to_sequential(oracle, n):
     assert np.all(np.diff(got) >= 0)
 
 
-def test_scan_repeated_runs_agree(oracle):
-    """The look-back publishes and polls tile descriptors across workgroups: 30 runs over 2442
-    tiles must all be exact (integer-valued input, reused workspace)."""
+def test_scan_repeated_runs_agree(oracle, scan_variant):
+    """Range sums travel between workgroups through the workspace (between two launches, or
+    published and polled inside one): 30 runs must all be exact (integer-valued input, reused
+    workspace)."""
     from gear_amd import ops
     n = 10_000_000
     rng = np.random.default_rng(5)
@@ -60,7 +76,7 @@ def test_scan_repeated_runs_agree(oracle):
     exp = torch.from_numpy(np.cumsum(p.astype(np.float64))).cuda()
     dp = _dev(p)
     out = torch.empty(n, dtype=torch.float64, device="cuda")
-    announce("scan repeated 30x n=%d" % n)
+    announce("scan repeated 30x n=%d %s" % (n, scan_variant))
     for it in range(30):
         out.fill_(-1.0)
         ops.prefix_sum(dp, out=out)
@@ -68,11 +84,11 @@ def test_scan_repeated_runs_agree(oracle):
 
 
 @pytest.mark.parametrize("n", [1, 2047, 2048, 2049, 100_000, 3_000_001])
-def test_scan_i64_exact(oracle, n):
+def test_scan_i64_exact(oracle, n, scan_variant):
     from gear_amd import ops
     rng = np.random.default_rng(n + 1)
     w = rng.integers(0, 1001, size=n).astype(np.int64)
-    announce("scan int64 n=%d" % n)
+    announce("scan int64 n=%d %s" % (n, scan_variant))
     got = ops.prefix_sum_i64(_dev(w)).cpu().numpy()
     assert np.array_equal(got, oracle.scan_i64(w))
     assert np.array_equal(got, np.cumsum(w))
