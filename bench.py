@@ -160,6 +160,34 @@ def run_config4(args):
     payload = B * span * sum(tab.step_bytes)
     alg_bytes = 2 * payload  # every gathered byte is read once and written once
     achieved = alg_bytes / (gather_ms * 1e-3) / 1e9
+
+    # Yardsticks of the same run: the batch payload moved as ONE contiguous piece, by the library's
+    # slice kernel and by torch's device-to-device copy.  What a plain copy reaches on this box is
+    # the practical ceiling of the gather; the roofline stays priced against the nominal peak.
+    yard = None
+    if not args.no_pipelined:
+        ydst = torch.empty(payload, dtype=torch.uint8, device="cuda")
+        ysrc = table[:payload]
+        zero = torch.zeros(1, dtype=torch.int64, device="cuda")
+
+        def timed_ms(fn, reps=20):
+            for _ in range(3):
+                fn()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / reps
+
+        ms_lib = timed_ms(lambda: ops.copy(table, ydst, zero, zero, payload))
+        ms_torch = timed_ms(lambda: ydst.copy_(ysrc))
+        yard = {"contiguous_copy_slice_kernel_GBps": alg_bytes / (ms_lib * 1e-3) / 1e9,
+                "contiguous_copy_torch_GBps": alg_bytes / (ms_torch * 1e-3) / 1e9,
+                "gather_vs_contiguous_copy": ms_lib / gather_ms,
+                "what": "%d bytes read + written as one contiguous piece, same run" % payload}
+        del ydst
     result = {
         "metric": "sampled windows/sec + gather GB/s (% of HBM peak) at batch 2048, 1 MI355X",
         "value": B / (ms_per_step * 1e-3),
@@ -177,6 +205,7 @@ def run_config4(args):
             "ms_per_step": ms_pipelined, "value": B / (ms_pipelined * 1e-3),
             "frac_of_hbm_peak": alg_bytes / (ms_pipelined * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "what": "same steps, sampler of batch i+1 on a second stream during gather i"},
+        "yardsticks": yard,
         "step_GBps": alg_bytes / (ms_per_step * 1e-3) / 1e9,
         "step_frac_of_hbm_peak": alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": achieved,
@@ -557,7 +586,7 @@ def main():
                     help="config 5: trajectories of 1000 steps in pinned host memory (2000 = 56.5 GB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-pipelined", action="store_true",
-                    help="config 4: skip the second, pipelined pass over the same steps")
+                    help="config 4: skip the pipelined pass over the same steps and the copy yardsticks")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB plain copies (slices kernel) before the steps")
     ap.add_argument("--traffic-bytes", type=float, default=None,
