@@ -307,6 +307,35 @@ def _time_steps(torch, step, steps, warmup, events=None):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def _time_graph(torch, body, feed, steps, warmup):
+    """The same steps replayed from a HIP graph (what a launch-bound loop wants): body() reads
+    static input buffers, feed(i) copies step i's inputs into them (eager, one small launch)."""
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):   # warm-up on the capture stream: workspaces get allocated
+        feed(0)
+        body()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        body()
+    for i in range(warmup):
+        feed(i)
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        feed(warmup + i)
+        graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def _graph_extra(B, unit, gms_):
+    return {"graph_replay": {"ms_per_step": gms_, "value": B / (gms_ * 1e-3), "unit": unit,
+                             "what": "same steps: inputs copied into static buffers, then one "
+                                     "replay of the captured step"}}
+
+
 def _line(metric_value, unit, args, ms, workload, roofline, extra=None):
     d = {"metric": "sampled windows/sec + gather GB/s (% of HBM peak) at batch 2048, 1 MI355X",
          "value": metric_value, "unit": unit, "n_gpus": 1, "steps": args.steps,
@@ -349,6 +378,11 @@ def run_config1(args):
 
     ms = _time_steps(torch, step, args.steps, args.warmup)
     gms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    cur = torch.empty(B, dtype=torch.int64, device="cuda")
+    ms_graph = _time_graph(
+        torch, lambda: ops.subcopy_multi(table, ops.sort_i64(cur, key_bits=12), tss, lens,
+                                         tab.traj_stride, cols),
+        lambda i: cur.copy_(draws[i]), args.steps, args.warmup)
     alg = 2 * B * tab.traj_stride
     host = table.cpu().numpy()
     hd = [np.zeros((B, 64 * sb), np.uint8) for sb in tab.step_bytes]
@@ -368,9 +402,10 @@ def run_config1(args):
                  {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": alg / (gms * 1e-3) / 1e9,
                   "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (gms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                   "avg_launch_ms": gms, "algorithmic_bytes": alg, "traffic": None},
-                 {"cpu_baseline": {"value": B / (cpu_ms * 1e-3), "unit": "trajectories/s", "cores": 1,
-                                   "kind": "port", "ms_per_step": cpu_ms,
-                                   "sample": "%d steps of sort + 4-column memset+memcpy gather" % n}})
+                 dict(_graph_extra(B, "trajectories/s", ms_graph),
+                      cpu_baseline={"value": B / (cpu_ms * 1e-3), "unit": "trajectories/s",
+                                    "cores": 1, "kind": "port", "ms_per_step": cpu_ms,
+                                    "sample": "%d steps of sort + 4-column memset+memcpy gather" % n}))
 
 
 def run_config2(args):
@@ -403,6 +438,14 @@ def run_config2(args):
 
     ms = _time_steps(torch, step, args.steps, args.warmup)
     sms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    ucur = torch.empty(B, dtype=torch.float32, device="cuda")
+
+    def body():
+        ops.prefix_sum(dpri, out=prefix)
+        ops.upper_bound(prefix, ucur, unit_uniforms=True, idx_out=idx, priorities=dpri, beta=0.4,
+                        weights_out=w)
+
+    ms_graph = _time_graph(torch, body, lambda i: ucur.copy_(u01[i]), args.steps, args.warmup)
     alg = 12 * n
     t0 = time.perf_counter()
     k = 0
@@ -419,9 +462,10 @@ def run_config2(args):
                  {"bound": "hbm", "kernel": "scan_init_kernel + scan_kernel", "achieved": alg / (sms * 1e-3) / 1e9,
                   "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (sms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                   "avg_launch_ms": sms, "algorithmic_bytes": alg, "traffic": None},
-                 {"cpu_baseline": {"value": B / (cpu_ms * 1e-3), "unit": "draws/s", "cores": 1,
-                                   "kind": "port", "ms_per_step": cpu_ms,
-                                   "sample": "%d steps of fp64 scan + 4096 searches + weights" % k}})
+                 dict(_graph_extra(B, "draws/s", ms_graph),
+                      cpu_baseline={"value": B / (cpu_ms * 1e-3), "unit": "draws/s", "cores": 1,
+                                    "kind": "port", "ms_per_step": cpu_ms,
+                                    "sample": "%d steps of fp64 scan + 4096 searches + weights" % k}))
 
 
 def run_config3(args):
@@ -463,13 +507,28 @@ def run_config3(args):
 
     ms = _time_steps(torch, step, args.steps, args.warmup)
     gms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    uc = torch.empty((2, B), dtype=torch.float64, device="cuda")
+
+    def body():
+        ops.prefix_sum_i64(lengths, out=prefix)
+        traj = ops.sort_i64(ops.upper_bound_i64(prefix, uc[0], unit_uniforms=True), key_bits=17)
+        lens = ops.take_i64(lengths, traj)
+        start = (uc[1] * (lens - (span - 1)).double()).long()
+        ops.subcopy_multi(table, traj, start, lens, tab.traj_stride, cols)
+
+    def feed(i):
+        uc[0].copy_(u1[i])
+        uc[1].copy_(u2[i])
+
+    ms_graph = _time_graph(torch, body, feed, args.steps, args.warmup)
     alg = 2 * B * span * sum(tab.step_bytes) + B * span
     return _line(B / (ms * 1e-3), "windows/s", args, ms,
                  "config3: %d variable-length trajectories (T=1000), length-weighted int64 sampler, "
                  "1024 windows x 20 steps x 5 columns + uint8 mask" % tab.capacity,
                  {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": alg / (gms * 1e-3) / 1e9,
                   "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (gms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                  "avg_launch_ms": gms, "algorithmic_bytes": alg, "traffic": None})
+                  "avg_launch_ms": gms, "algorithmic_bytes": alg, "traffic": None},
+                 _graph_extra(B, "windows/s", ms_graph))
 
 
 def run_config5(args):
