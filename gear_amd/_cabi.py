@@ -43,6 +43,9 @@ SIGNATURES = {
                                  c_void_p]),
     "gear_hip_subcopy_multi": (c_int, [c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_i64,
                                        ctypes.POINTER(ColumnDesc), c_int, c_void_p]),
+    "gear_hip_subcopy_multi_checked": (c_int, [c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_i64,
+                                               c_i64, c_i64, ctypes.POINTER(ColumnDesc), c_int,
+                                               c_void_p]),
     "gear_hip_vcopy": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_i64,
                                c_void_p]),
     "gear_hip_copy": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_i64, c_void_p]),

@@ -45,6 +45,8 @@ struct GatherArgs {
   const int64_t *c;  // subcopy: lens        vcopy: strides
   int64_t traj_stride;
   int64_t fixed_stride;  // copy mode
+  int64_t capacity;      // subcopy: trajectories in the table, 0 = indices are not checked
+  int64_t traj_len;      // subcopy: steps per trajectory, 0 = lengths are not clamped
 };
 
 struct MultiArgs {
@@ -138,7 +140,10 @@ __device__ __forceinline__ void gather_chunks(const Slice &s, int64_t c, int64_t
 // Window arithmetic of fused_subcopy_collect (src/cuda/copy.cu:110-123) in int64.
 __device__ __forceinline__ Slice resolve_window(const GatherArgs &p, const ColumnArgs &col,
                                                 int64_t g, int64_t *valid_steps) {
-  const int64_t idx = p.a[g], ts = p.b[g], len = p.c[g];
+  const int64_t idx = p.a[g], ts = p.b[g];
+  int64_t len = p.c[g];
+  if (p.traj_len > 0 && len > p.traj_len) len = p.traj_len;
+  if (p.capacity > 0 && (idx < 0 || idx >= p.capacity)) len = 0;  // nothing to read: all padding
   int64_t lsub = ts + col.ofst;
   if (lsub < 0) lsub = 0;
   int64_t rsub = lsub + col.span;
@@ -431,7 +436,7 @@ extern "C" int gear_hip_subcopy(const void *src, void *dst, int64_t num, const i
   int rc = fill_column(d, num, U, &col, &blocks);
   if (rc) return rc;
   if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
-  GatherArgs p{static_cast<const uint8_t *>(src), num, idxs, tss, lens, traj_stride, 0};
+  GatherArgs p{static_cast<const uint8_t *>(src), num, idxs, tss, lens, traj_stride, 0, 0, 0};
   return launch_subcopy(p, col, blocks, U, pick_nt(), as_stream(stream));
 }
 
@@ -439,7 +444,18 @@ extern "C" int gear_hip_subcopy_multi(const void *src, int64_t num, const int64_
                                       const int64_t *tss, const int64_t *lens,
                                       int64_t traj_stride, const gear_hip_column_desc *cols,
                                       int ncols, void *stream) {
-  if (num < 0 || ncols < 0 || ncols > GEAR_HIP_MAX_COLUMNS) return GEAR_HIP_EINVAL;
+  return gear_hip_subcopy_multi_checked(src, num, idxs, tss, lens, traj_stride, 0, 0, cols, ncols,
+                                        stream);
+}
+
+extern "C" int gear_hip_subcopy_multi_checked(const void *src, int64_t num, const int64_t *idxs,
+                                              const int64_t *tss, const int64_t *lens,
+                                              int64_t traj_stride, int64_t capacity,
+                                              int64_t trajectory_length,
+                                              const gear_hip_column_desc *cols, int ncols,
+                                              void *stream) {
+  if (num < 0 || ncols < 0 || ncols > GEAR_HIP_MAX_COLUMNS || capacity < 0 || trajectory_length < 0)
+    return GEAR_HIP_EINVAL;
   if (num == 0 || ncols == 0) return 0;
   if (!src || !idxs || !tss || !lens || !cols || traj_stride < 0) return GEAR_HIP_EINVAL;
   const int U = pick_unroll();
@@ -455,7 +471,8 @@ extern "C" int gear_hip_subcopy_multi(const void *src, int64_t num, const int64_
   }
   for (int i = ncols; i < GEAR_HIP_MAX_COLUMNS; ++i) m.col[i] = m.col[0];
   if (total >= 0x7fffffffll) return GEAR_HIP_ERANGE;
-  GatherArgs p{static_cast<const uint8_t *>(src), num, idxs, tss, lens, traj_stride, 0};
+  GatherArgs p{static_cast<const uint8_t *>(src), num,        idxs, tss, lens, traj_stride, 0,
+               capacity,                          trajectory_length};
   return launch_multi(p, m, total, U, pick_nt(), as_stream(stream));
 }
 
@@ -465,7 +482,7 @@ extern "C" int gear_hip_vcopy(const void *src, void *dst, int64_t num,
   if (num < 0 || max_stride < 0) return GEAR_HIP_EINVAL;
   if (num == 0) return 0;
   if (!src || !dst || !src_offsets || !dst_offsets || !strides) return GEAR_HIP_EINVAL;
-  GatherArgs p{static_cast<const uint8_t *>(src), num, src_offsets, dst_offsets, strides, 0, 0};
+  GatherArgs p{static_cast<const uint8_t *>(src), num, src_offsets, dst_offsets, strides, 0, 0, 0, 0};
   return launch_slices<kVcopy>(p, static_cast<uint8_t *>(dst), max_stride, as_stream(stream));
 }
 
@@ -475,7 +492,7 @@ extern "C" int gear_hip_copy(const void *src, void *dst, int64_t num, const int6
   if (num == 0 || stride == 0) return 0;
   if (!src || !dst || !src_offsets || !dst_offsets) return GEAR_HIP_EINVAL;
   GatherArgs p{static_cast<const uint8_t *>(src), num, src_offsets, dst_offsets, nullptr, 0,
-               stride};
+               stride, 0, 0};
   return launch_slices<kCopy>(p, static_cast<uint8_t *>(dst), stride, as_stream(stream));
 }
 

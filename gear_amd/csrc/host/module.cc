@@ -499,12 +499,13 @@ PYBIND11_MODULE(_libgear, libgear) {
                descs[k].zero_fill = zero_fill ? 1 : 0;
              }
              check_hip("subcopy_multi",
-                       gear_hip_subcopy_multi(h.impl.device_base(), a.numel,
-                                              static_cast<const int64_t *>(a.ptr),
-                                              static_cast<const int64_t *>(b.ptr),
-                                              static_cast<const int64_t *>(c.ptr),
-                                              (int64_t)h.impl.table().trajectory_stride(), descs.data(),
-                                              (int)descs.size(), current_stream()));
+                       gear_hip_subcopy_multi_checked(
+                           h.impl.device_base(), a.numel, static_cast<const int64_t *>(a.ptr),
+                           static_cast<const int64_t *>(b.ptr), static_cast<const int64_t *>(c.ptr),
+                           (int64_t)h.impl.table().trajectory_stride(),
+                           (int64_t)h.impl.table().table_spec().capacity,
+                           (int64_t)h.impl.table().table_spec().trajectory_length, descs.data(),
+                           (int)descs.size(), current_stream()));
            },
            py::arg("indices"), py::arg("timesteps"), py::arg("lengths"), py::arg("columns"),
            py::arg("dsts"), py::arg("zero_fill") = true, py::arg("masks") = py::none())

@@ -93,11 +93,13 @@ def subcopy(src, dst, idxs, tss, lens, *, pad_head, ofst, span, traj_stride, ste
     return dst
 
 
-def subcopy_multi(src, idxs, tss, lens, traj_stride, columns):
+def subcopy_multi(src, idxs, tss, lens, traj_stride, columns, capacity=0, trajectory_length=0):
     """All columns of one batch in one launch.
 
     columns: list of dicts with keys dst, ofst, span, step_bytes, col_base, pad_head and
     optionally zero_fill (default True), mask_out, dst_stride.
+    capacity / trajectory_length > 0: the kernel checks every window against the table (an index
+    outside [0, capacity) gathers nothing, lens are clamped to trajectory_length).
     """
     _need(idxs, torch.int64, "idxs")
     _need(tss, torch.int64, "tss")
@@ -126,8 +128,8 @@ def subcopy_multi(src, idxs, tss, lens, traj_stride, columns):
         descs[i].dst_stride = int(stride)
         descs[i].pad_head = int(bool(c["pad_head"]))
         descs[i].zero_fill = int(bool(c.get("zero_fill", True)))
-    call("gear_hip_subcopy_multi", _src_ptr(src), num, _ptr(idxs), _ptr(tss), _ptr(lens),
-         int(traj_stride), descs, n, _stream())
+    call("gear_hip_subcopy_multi_checked", _src_ptr(src), num, _ptr(idxs), _ptr(tss), _ptr(lens),
+         int(traj_stride), int(capacity), int(trajectory_length), descs, n, _stream())
 
 
 def vcopy(src, dst, src_offsets, dst_offsets, strides, max_stride):

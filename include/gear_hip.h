@@ -122,6 +122,17 @@ int gear_hip_subcopy_multi(const void *src, int64_t num, const int64_t *idxs, co
                            const int64_t *lens, int64_t traj_stride,
                            const gear_hip_column_desc *cols, int ncols, void *stream);
 
+/* The same launch with the batch checked against the table on the device: a window whose
+ * trajectory index lies outside [0, capacity) reads nothing (its rows are all padding, its mask
+ * all 0) and lens[g] is clamped to trajectory_length, so no index a caller passes can make the
+ * kernel read outside the table.  The reference's kernel trusts its inputs
+ * (src/cuda/copy.cu:110-123); capacity = 0 / trajectory_length = 0 switch the respective check
+ * off, which is what gear_hip_subcopy_multi does. */
+int gear_hip_subcopy_multi_checked(const void *src, int64_t num, const int64_t *idxs,
+                                   const int64_t *tss, const int64_t *lens, int64_t traj_stride,
+                                   int64_t capacity, int64_t trajectory_length,
+                                   const gear_hip_column_desc *cols, int ncols, void *stream);
+
 /* Generic slice gather: dst[dst_offsets[g] .. +strides[g]) = src[src_offsets[g] .. +strides[g]).
  * Replaces launch_vary_stride_copy_collect / vary_stride_copy_collect
  * (src/cuda/copy.cu:47-89,175-215; libgear.core.vcopy / copy_debug, copy.cu:247-258).

@@ -169,6 +169,45 @@ def test_odd_byte_columns_every_alignment(oracle):
                 assert np.array_equal(mask, rmask)
 
 
+def test_checked_gather_ignores_indices_outside_the_table(oracle):
+    """gear_hip_subcopy_multi_checked: trajectory indices outside [0, capacity) gather nothing (all
+    padding, mask 0) and lengths beyond the trajectory length are clamped, so a bad batch cannot
+    make the kernel read outside the table.  Expected = the oracle on the sanitised batch."""
+    from gear_amd import ops
+    schema = Schema(CFG3, T=50, capacity=40)
+    table = fill_random(schema, 9)
+    rng = np.random.default_rng(9)
+    B, span = 300, 20
+    idxs = rng.integers(0, 40, size=B).astype(np.int64)
+    lens = rng.integers(1, 51, size=B).astype(np.int64)
+    tss = (rng.integers(0, 1 << 20, size=B) % lens).astype(np.int64)
+    idxs[::7] = -1 - rng.integers(0, 1 << 40, size=len(idxs[::7]))
+    idxs[3::7] = 40 + rng.integers(0, 1 << 40, size=len(idxs[3::7]))
+    lens[5::11] = 51 + rng.integers(0, 1 << 30, size=len(lens[5::11]))
+    bad = (idxs < 0) | (idxs >= 40)
+    s_idx = np.where(bad, 0, idxs)
+    s_len = np.where(bad, 0, np.minimum(lens, 50))
+    tdev = _dev(table)
+    for pad_head in (False, True):
+        dsts = [torch.full((B, span * sb), 0xCD, dtype=torch.uint8, device="cuda")
+                for sb in schema.step_bytes]
+        masks = [torch.full((B, span), 9, dtype=torch.uint8, device="cuda") for _ in range(5)]
+        cols = [dict(dst=dsts[c], ofst=-5, span=span, step_bytes=schema.step_bytes[c],
+                     col_base=schema.col_base(c), pad_head=pad_head, mask_out=masks[c])
+                for c in range(5)]
+        announce("checked multi-column gather pad_head=%s" % pad_head)
+        ops.subcopy_multi(tdev, _dev(idxs), _dev(tss), _dev(lens), schema.traj_stride, cols,
+                          capacity=40, trajectory_length=50)
+        torch.cuda.synchronize()
+        for c in range(5):
+            exp, emask = oracle.subcopy(table, s_idx, tss, s_len, pad_head, -5, span,
+                                        schema.traj_stride, schema.step_bytes[c],
+                                        schema.col_base(c), want_mask=True)
+            assert np.array_equal(dsts[c].cpu().numpy(), exp)
+            assert np.array_equal(masks[c].cpu().numpy(), emask)
+        assert not dsts[0].cpu().numpy()[bad].any() and not masks[0].cpu().numpy()[bad].any()
+
+
 def test_empty_batch():
     from gear_amd import ops
     t = torch.zeros(1024, dtype=torch.uint8, device="cuda")
