@@ -218,25 +218,28 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
 // ---- one-workgroup sort for small batches (a sampled batch of indices) --------------------------
 // Up to kSmallMax keys stay in registers (element e = r*1024 + tid, r < 4) and move through LDS
 // once per digit.  Ballots rank equal digits inside a wave; a digit-major table of
-// (digit, round*16+wave) counts, one counter per thread, is scanned by the workgroup.  The table
-// has 1024 counters, so the digit is 6 bits wide for up to 1024 keys, 5 bits up to 2048 and
-// 4 bits up to 4096.  The payload is carried as the element's original position.
+// (digit, round*16+wave) counts, four counters per thread, is scanned by the workgroup.  The table
+// has 4096 counters, so the digit is 8 bits wide for up to 1024 keys, 7 bits up to 2048 and
+// 6 bits up to 4096.  One workgroup runs on one CU, where every instruction of the 16 waves costs
+// issue time: the payload (the element's original position) is carried only where it is needed.
 constexpr int kSmallBlock = 1024;
 constexpr int kSmallRounds = 4;
 constexpr int kSmallMax = kSmallBlock * kSmallRounds;
 constexpr int kSmallWaves = kSmallBlock / kWave;
+constexpr int kSmallCounters = 4 * kSmallBlock;
 
 template <typename K>
 struct SmallSortSmem {
   K kbuf[kSmallMax];
   uint16_t pbuf[kSmallMax];
-  uint32_t cnt[kSmallBlock];
+  uint32_t cnt[kSmallCounters];
   uint32_t wsum[kSmallWaves];
 };
 
 // Sorts bits [begin_bit, end_bit) of the keys held by the workgroup, stable; on return key[r] /
-// perm[r] of thread tid are the key and original position of sorted element r*1024 + tid.
-template <typename K>
+// perm[r] (HAS_PERM) of thread tid are the key and original position of sorted element
+// r*1024 + tid.
+template <typename K, bool HAS_PERM>
 __device__ __forceinline__ void block_sort_small(K (&key)[kSmallRounds],
                                                  uint32_t (&perm)[kSmallRounds], int num,
                                                  int begin_bit, int end_bit,
@@ -244,9 +247,10 @@ __device__ __forceinline__ void block_sort_small(K (&key)[kSmallRounds],
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
   const int nr = (num + kSmallBlock - 1) / kSmallBlock;  // active rounds, 1..4
-  const int dbits = nr <= 1 ? 6 : (nr == 2 ? 5 : 4);
+  const int dbits = nr <= 1 ? 8 : (nr == 2 ? 7 : 6);
   const int slots = nr * kSmallWaves;
-  sm.cnt[tid] = 0;
+  u32x4 *cnt4 = reinterpret_cast<u32x4 *>(sm.cnt);
+  cnt4[tid] = u32x4{0u, 0u, 0u, 0u};
   __syncthreads();
   for (int shift = begin_bit; shift < end_bit; shift += dbits) {
     const int width = end_bit - shift >= dbits ? dbits : end_bit - shift;
@@ -270,21 +274,30 @@ __device__ __forceinline__ void block_sort_small(K (&key)[kSmallRounds],
       }
     }
     __syncthreads();
-    // exclusive scan of the counters, one per thread
-    const int c = (int)sm.cnt[tid];
-    const int inc = wave_inclusive_sum(c);
-    if (lane == 63) sm.wsum[wave] = (uint32_t)inc;
-    __syncthreads();
-    uint32_t before = 0;
-    for (int w = 0; w < wave; ++w) before += sm.wsum[w];
-    sm.cnt[tid] = before + (uint32_t)(inc - c);
+    // exclusive scan of the counters, four consecutive ones per thread
+    {
+      const u32x4 c = cnt4[tid];
+      const int s4 = (int)(c[0] + c[1] + c[2] + c[3]);
+      const int inc = wave_inclusive_sum(s4);
+      if (lane == 63) sm.wsum[wave] = (uint32_t)inc;
+      __syncthreads();
+      const int wtot = lane < kSmallWaves ? (int)sm.wsum[lane] : 0;
+      const int winc = wave_inclusive_sum(wtot);
+      const uint32_t before = wave == 0 ? 0u : (uint32_t)wave_read_lane(winc, wave - 1);
+      u32x4 e;
+      e[0] = before + (uint32_t)(inc - s4);
+      e[1] = e[0] + c[0];
+      e[2] = e[1] + c[1];
+      e[3] = e[2] + c[2];
+      cnt4[tid] = e;
+    }
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < kSmallRounds; ++r) {
       if (r < nr && r * kSmallBlock + tid < num) {
         const uint32_t pos = sm.cnt[slot[r]] + (uint32_t)rank[r];
         sm.kbuf[pos] = key[r];
-        sm.pbuf[pos] = (uint16_t)perm[r];
+        if (HAS_PERM) sm.pbuf[pos] = (uint16_t)perm[r];
       }
     }
     __syncthreads();
@@ -293,10 +306,10 @@ __device__ __forceinline__ void block_sort_small(K (&key)[kSmallRounds],
       const int e = r * kSmallBlock + tid;
       if (r < nr && e < num) {
         key[r] = sm.kbuf[e];
-        perm[r] = sm.pbuf[e];
+        if (HAS_PERM) perm[r] = sm.pbuf[e];
       }
     }
-    sm.cnt[tid] = 0;
+    cnt4[tid] = u32x4{0u, 0u, 0u, 0u};
     __syncthreads();
   }
 }
@@ -317,7 +330,7 @@ __global__ __launch_bounds__(kSmallBlock) void small_sort_kernel(const K *__rest
     key[r] = e < num ? kin[e] : (K)0;
     perm[r] = (uint32_t)e;
   }
-  block_sort_small<K>(key, perm, num, begin_bit, end_bit, sm);
+  block_sort_small<K, HAS_V>(key, perm, num, begin_bit, end_bit, sm);
 #pragma unroll
   for (int r = 0; r < kSmallRounds; ++r) {
     const int e = r * kSmallBlock + tid;

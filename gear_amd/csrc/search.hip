@@ -101,21 +101,23 @@ __global__ __launch_bounds__(kBlock) void search_i64_kernel(const int64_t *__res
 // One workgroup: sort the found indices in LDS and split them into window arguments.  (The
 // search itself stays a many-workgroup kernel: its probes are divergent loads, and one CU issues
 // only about one cache line per clock.)
+// K: uint32_t where every index fits (prefix shorter than 2^32 entries), else uint64_t.
+template <typename K>
 __global__ __launch_bounds__(radix::kSmallBlock) void sort_split_small_kernel(
     const int64_t *__restrict__ raw, int num, int key_bits, int64_t *__restrict__ sorted_out,
     int64_t T, int64_t modulo, int64_t *__restrict__ idxs, int64_t *__restrict__ tss,
     int64_t *__restrict__ lens) {
-  __shared__ radix::SmallSortSmem<uint64_t> sm;
+  __shared__ radix::SmallSortSmem<K> sm;
   const int tid = threadIdx.x;
-  uint64_t key[radix::kSmallRounds];
+  K key[radix::kSmallRounds];
   uint32_t perm[radix::kSmallRounds];
 #pragma unroll
   for (int r = 0; r < radix::kSmallRounds; ++r) {
     const int e = r * radix::kSmallBlock + tid;
-    key[r] = e < num ? (uint64_t)raw[e] : 0ull;
-    perm[r] = (uint32_t)e;
+    key[r] = e < num ? (K)raw[e] : (K)0;
+    perm[r] = 0u;
   }
-  radix::block_sort_small<uint64_t>(key, perm, num, 0, key_bits, sm);
+  radix::block_sort_small<K, false>(key, perm, num, 0, key_bits, sm);
 #pragma unroll
   for (int r = 0; r < radix::kSmallRounds; ++r) {
     const int e = r * radix::kSmallBlock + tid;
@@ -123,9 +125,18 @@ __global__ __launch_bounds__(radix::kSmallBlock) void sort_split_small_kernel(
       int64_t f = (int64_t)key[r];
       if (sorted_out) sorted_out[e] = f;
       if (T > 0) {
-        if (modulo > 0) f %= modulo;
-        const int64_t traj = f / T;
-        const int64_t ts = f - traj * T;
+        int64_t traj, ts;
+        if (sizeof(K) == 4 && T <= 0xffffffffll && modulo <= 0xffffffffll) {
+          uint32_t f32 = (uint32_t)key[r];  // 32-bit division is a fraction of the 64-bit one
+          if (modulo > 0) f32 %= (uint32_t)modulo;
+          const uint32_t q = f32 / (uint32_t)T;
+          traj = q;
+          ts = f32 - q * (uint32_t)T;
+        } else {
+          if (modulo > 0) f %= modulo;
+          traj = f / T;
+          ts = f - traj * T;
+        }
         idxs[e] = traj;
         tss[e] = ts;
         if (lens) lens[e] = ts + 1;
@@ -251,8 +262,12 @@ extern "C" int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const
       prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   if (num <= radix::kSmallMax) {
-    sort_split_small_kernel<<<dim3(1), dim3(radix::kSmallBlock), 0, st>>>(
-        raw, (int)num, key_bits, sorted_out, trajectory_length, modulo, idxs, tss, lens);
+    if (n <= (1ll << 32))
+      sort_split_small_kernel<uint32_t><<<dim3(1), dim3(radix::kSmallBlock), 0, st>>>(
+          raw, (int)num, key_bits, sorted_out, trajectory_length, modulo, idxs, tss, lens);
+    else
+      sort_split_small_kernel<uint64_t><<<dim3(1), dim3(radix::kSmallBlock), 0, st>>>(
+          raw, (int)num, key_bits, sorted_out, trajectory_length, modulo, idxs, tss, lens);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
