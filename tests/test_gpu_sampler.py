@@ -236,3 +236,23 @@ def test_sample_sorted_equals_search_then_sort(oracle, num):
     assert np.array_equal(idxs.cpu().numpy(), f // T)
     assert np.array_equal(tss.cpu().numpy(), f % T)
     assert np.array_equal(lens.cpu().numpy(), f % T + 1)
+
+
+@pytest.mark.parametrize("num", [64, 65, 2048, 4096])
+def test_sample_sorted_with_many_equal_indices(oracle, num):
+    """Few buckets, many draws: nearly every found index repeats, so the ranking sort must place
+    equal keys by position without gaps or collisions."""
+    from gear_amd import ops
+    n, T = 37, 5
+    p = _priorities(n, 5)
+    u01 = np.random.default_rng(num + 1).random(num, dtype=np.float32)
+    announce("sample_sorted ties num=%d" % num)
+    prefix = ops.prefix_sum(_dev(p))
+    srt, idxs, tss, lens = ops.sample_sorted(prefix, _dev(u01), unit_uniforms=True,
+                                             trajectory_length=T)
+    torch.cuda.synchronize()
+    exp = np.sort(oracle.upper_bound_f64(prefix.cpu().numpy(), u01, unit_uniforms=True))
+    assert np.array_equal(srt.cpu().numpy(), exp)
+    assert np.array_equal(idxs.cpu().numpy(), exp // T)
+    assert np.array_equal(tss.cpu().numpy(), exp % T)
+    assert np.array_equal(lens.cpu().numpy(), exp % T + 1)
