@@ -98,80 +98,19 @@ __global__ __launch_bounds__(kBlock) void search_i64_kernel(const int64_t *__res
   idx_out[j] = i;
 }
 
-// Sort of a small batch of found indices by ranking, fused with the split into window arguments.
-// Every workgroup keeps ALL keys of the batch in LDS and ranks 64 of them: rank(e) = number of
-// keys smaller than key e, plus equal keys at smaller positions (the order of a stable sort).  The
-// sixteen waves of a workgroup each count over a sixteenth of the keys (a lone wave per SIMD
-// issues a dependent instruction only every ~8 clocks, so the CU wants several); a key read from
-// LDS is broadcast to the 64 lanes and costs a compare and an add per lane.  num / 64
-// workgroups run side by side on as many CUs, where a one-workgroup radix sort of the same batch
-// is bound by the instruction issue of a single CU (11 us against ~6 us for 2048 keys).
-// Used for prefixes shorter than 2^32 entries (K = uint32_t); longer ones take the radix sort.
-constexpr int kRankBlock = 1024;
-constexpr int kRankWaves = kRankBlock / kWave;
-constexpr int kRankMax = radix::kSmallMax;
-
-template <typename K>
-__global__ __launch_bounds__(kRankBlock) void rank_split_kernel(
+// The ranking sort of radix_sort.hpp over the found indices, fused with the split into window
+// arguments.  Used for prefixes shorter than 2^32 entries (the compare key is the index as
+// uint32_t); longer ones take the radix sort.
+__global__ __launch_bounds__(radix::kRankBlock) void rank_split_kernel(
     const int64_t *__restrict__ raw, int num, int64_t *__restrict__ sorted_out, int64_t T,
     int64_t modulo, int64_t *__restrict__ idxs, int64_t *__restrict__ tss,
     int64_t *__restrict__ lens) {
-  __shared__ K keys[kRankMax];
-  __shared__ uint32_t part[kRankWaves][kWave];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int padded = (num + 16 * kRankWaves - 1) & ~(16 * kRankWaves - 1);  // wave shares: multiples of 16 keys
-  {
-    // all of a thread's loads are issued before the first LDS write (one memory round trip)
-    constexpr int kPerThread = kRankMax / kRankBlock;
-    K mykeys[kPerThread];
-#pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const int j = tid + i * kRankBlock;
-      mykeys[i] = j < num ? (K)raw[j] : (K)~(K)0;
-    }
-#pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const int j = tid + i * kRankBlock;
-      if (j < padded) keys[j] = mykeys[i];
-    }
-  }
-  __syncthreads();
-  const int e0 = (int)blockIdx.x * kWave, e = e0 + lane;
-  const K mine = keys[e < num ? e : 0];
-  const int share = padded / kRankWaves;
-  const int jb = wave * share, je = jb + share;
-  uint32_t c = 0;
-  // three stretches with a uniform rule each, sixteen keys (four LDS reads in flight) per step
-  const int before_end = je < e0 ? je : (e0 > jb ? e0 : jb);
-  for (int j = jb; j < before_end; j += 16) {  // positions before this workgroup's keys
-    K k[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) k[i] = keys[j + i];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) c += k[i] <= mine;  // equal keys at smaller positions rank first
-  }
-  const int in_begin = jb > e0 ? jb : e0, in_end = je < e0 + kWave ? je : e0 + kWave;
-  for (int j = in_begin; j < in_end; j += 16) {
-    K k[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) k[i] = keys[j + i];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) c += (k[i] < mine) || (k[i] == mine && j + i < e);
-  }
-  const int after_begin = jb > e0 + kWave ? jb : (e0 + kWave < je ? e0 + kWave : je);
-  for (int j = after_begin; j < je; j += 16) {
-    K k[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) k[i] = keys[j + i];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) c += k[i] < mine;
-  }
-  part[wave][lane] = c;
-  __syncthreads();
-  if (wave != 0 || e >= num) return;
-  uint32_t rank = 0;
-#pragma unroll
-  for (int w = 0; w < kRankWaves; ++w) rank += part[w][lane];
+  typedef uint32_t K;
+  __shared__ radix::RankSmem<K> sm;
+  K mine;
+  const uint32_t rank = radix::block_rank<K>(sm, num, [&](int j) { return (K)raw[j]; }, &mine);
+  const int e = (int)blockIdx.x * kWave + (threadIdx.x & 63);
+  if (threadIdx.x >= kWave || e >= num) return;
   int64_t f = (int64_t)mine;
   if (sorted_out) sorted_out[rank] = f;
   if (T > 0) {
@@ -309,8 +248,8 @@ extern "C" int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const
   search_f64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(
       prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  if (num <= kRankMax && n < (1ll << 32)) {
-    rank_split_kernel<uint32_t><<<dim3((unsigned)ceil_div64(num, kWave)), dim3(kRankBlock), 0, st>>>(
+  if (num <= radix::kRankMax && n < (1ll << 32)) {
+    rank_split_kernel<<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(
         raw, (int)num, sorted_out, trajectory_length, modulo, idxs, tss, lens);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
