@@ -111,15 +111,30 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
     const uint32_t *__restrict__ table, const uint32_t *__restrict__ totals,
     uint32_t *__restrict__ next, int next_shift, uint32_t next_dmask,
     uint32_t *__restrict__ clear) {
+  constexpr int kSub = 4;                  // rounds ranked together: independent ballot chains
+  constexpr int kSlots = kSub * kWaves;    // (round, wave) slots of the count table
   __shared__ uint32_t base[kBins];
-  __shared__ uint32_t wcnt[kWaves][kBins];
+  __shared__ uint32_t wcnt[kSlots][kBins];  // keys of digit d seen by slot s (kept zero between uses)
+  __shared__ uint32_t wpre[kSlots][kBins];  // where slot s starts writing digit d
   __shared__ uint32_t wsum[kWaves];
   __shared__ uint32_t part[FUSED ? kWaves : 1][2][kBins];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t tile = blockIdx.x;
-  // keys of the first round are loaded before the offsets are worked out
+  // keys of the first rounds are loaded before the offsets are worked out
   const int64_t tile0 = tile * kBlock * rounds;
-  K key = (tile0 + tid < num) ? kin[tile0 + tid] : (K)0;
+  K key[kSub];
+  V val[kSub];
+  auto load_rounds = [&](int r0) {
+#pragma unroll
+    for (int q = 0; q < kSub; ++q) {
+      const int64_t i = tile0 + (int64_t)(r0 + q) * kBlock + tid;
+      const bool ok = r0 + q < rounds && i < num;
+      key[q] = ok ? kin[i] : (K)0;
+      val[q] = V();
+      if (HAS_V && ok) val[q] = vin[i];
+    }
+  };
+  load_rounds(0);
   {
     uint32_t before = 0, total = 0;  // of digit tid: in the tiles before this one, in all tiles
     if (FUSED) {
@@ -163,7 +178,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
     const int inc = wave_inclusive_sum((int)total);
     if (lane == 63) wsum[wave] = (uint32_t)inc;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) wcnt[w][tid] = 0;
+    for (int w = 0; w < kSlots; ++w) wcnt[w][tid] = 0;
     __syncthreads();
     uint32_t lower = (uint32_t)inc - total;  // keys with a smaller digit
     for (int w = 0; w < wave; ++w) lower += wsum[w];
@@ -172,46 +187,61 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   __syncthreads();
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
   const int64_t tile_elems = (int64_t)kBlock * rounds;
-  for (int r = 0; r < rounds; ++r) {
-    const int64_t i = tile0 + (int64_t)r * kBlock + tid;
-    const bool valid = i < num;
-    V val = V();
-    if (HAS_V && valid) val = vin[i];
-    K key_next = (K)0;
-    if (r + 1 < rounds && i + kBlock < num) key_next = kin[i + kBlock];
-    const uint32_t d = (uint32_t)(key >> shift) & dmask;
-    uint64_t peers = wave_ballot(valid);
+  for (int r0 = 0; r0 < rounds; r0 += kSub) {
+    bool valid[kSub];
+    uint32_t d[kSub];
+    int rank[kSub];
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      const bool bit = (d >> b) & 1u;
-      const uint64_t bal = wave_ballot(bit);
-      peers &= bit ? bal : ~bal;
-    }
-    const int rank = __popcll(peers & lt_mask);
-    if (valid && rank == 0) wcnt[wave][d] = (uint32_t)__popcll(peers);
-    __syncthreads();
-    if (valid) {
-      uint32_t pos = base[d] + (uint32_t)rank;
-      for (int w = 0; w < wave; ++w) pos += wcnt[w][d];
-      kout[pos] = key;
-      if (HAS_V) vout[pos] = val;
-      if (FUSED && next)
-        atomicAdd(&next[(int64_t)(pos / tile_elems) * kBins +
-                        ((uint32_t)(key >> next_shift) & next_dmask)],
-                  1u);
+    for (int q = 0; q < kSub; ++q) {
+      const int64_t i = tile0 + (int64_t)(r0 + q) * kBlock + tid;
+      valid[q] = r0 + q < rounds && i < num;
+      d[q] = (uint32_t)(key[q] >> shift) & dmask;
+      uint64_t peers = wave_ballot(valid[q]);
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const bool bit = (d[q] >> b) & 1u;
+        const uint64_t bal = wave_ballot(bit);
+        peers &= bit ? bal : ~bal;
+      }
+      rank[q] = __popcll(peers & lt_mask);
+      if (valid[q] && rank[q] == 0) wcnt[q * kWaves + wave][d[q]] = (uint32_t)__popcll(peers);
     }
     __syncthreads();
     {
-      uint32_t s = 0;
+      // thread tid owns digit tid: running start over the slots in element order; the counts
+      // are cleared for the next use on the way
+      uint32_t run = base[tid];
 #pragma unroll
-      for (int w = 0; w < kWaves; ++w) {
-        s += wcnt[w][tid];
-        wcnt[w][tid] = 0;
+      for (int sl = 0; sl < kSlots; ++sl) {
+        const uint32_t c = wcnt[sl][tid];
+        wcnt[sl][tid] = 0;
+        wpre[sl][tid] = run;
+        run += c;
       }
-      base[tid] += s;
+      base[tid] = run;
     }
     __syncthreads();
-    key = key_next;
+    K kcur[kSub];
+    V vcur[kSub];
+#pragma unroll
+    for (int q = 0; q < kSub; ++q) {
+      kcur[q] = key[q];
+      vcur[q] = val[q];
+    }
+    if (r0 + kSub < rounds) load_rounds(r0 + kSub);  // in flight during the scatter
+#pragma unroll
+    for (int q = 0; q < kSub; ++q) {
+      if (valid[q]) {
+        const uint32_t pos = wpre[q * kWaves + wave][d[q]] + (uint32_t)rank[q];
+        kout[pos] = kcur[q];
+        if (HAS_V) vout[pos] = vcur[q];
+        if (FUSED && next)
+          atomicAdd(&next[(int64_t)(pos / tile_elems) * kBins +
+                          ((uint32_t)(kcur[q] >> next_shift) & next_dmask)],
+                    1u);
+      }
+    }
+    // the next use of wpre is ordered behind this scatter by the barrier after the next ballots
   }
 }
 
