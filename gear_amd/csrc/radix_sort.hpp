@@ -4,11 +4,11 @@
 // digits inside a wave, a small LDS table the rank across the waves of the tile) and scatters keys
 // and payloads to their final place for this digit.  Ranks follow element order, so the sort is
 // stable.  Where a key lands depends on a table of (tile, digit) counts:
-//  * up to kFusedTiles tiles (the candidate lists of top-k, index batches): one launch per digit.
-//    The table is tile-major; every workgroup sums the counts of the tiles before it and scans the
-//    digit totals itself, and while it scatters it counts the next digit of every key into the
-//    next table at the tile the key lands in (global atomics).  Three tables rotate: read, count,
-//    clear.  A first launch counts digit 0.
+//  * up to kFusedTiles tiles (the candidate lists of top-k, index batches): two launches per digit.
+//    A count launch fills a tile-major table; every scatter workgroup sums the counts of the tiles
+//    before it and scans the digit totals itself.  (Counting the next digit from inside the
+//    scatter launch with global atomics, one launch per digit, was measured too: 65 536 atomics
+//    cost 6.9 us per digit, the count launch 4.6 us.)
 //  * more tiles: count launch, one workgroup per digit scans its row of the digit-major table,
 //    scatter launch.
 #pragma once
@@ -26,7 +26,7 @@ constexpr int kFusedTiles = 128;
 struct Plan {
   int rounds;      // elements per thread and tile
   int64_t ntiles;  // tiles of kBlock * rounds elements
-  bool fused;      // one launch per digit
+  bool fused;      // the scatter workgroups sum the count table themselves
 };
 
 inline Plan plan(int64_t num) {
@@ -42,19 +42,17 @@ inline Plan plan(int64_t num) {
 
 inline size_t table_bytes(const Plan &p) { return (size_t)p.ntiles * kBins * sizeof(uint32_t); }
 
-// digit totals (1 KiB) followed by one table, or by three where the launches are fused
+// digit totals (1 KiB) followed by the count table
 inline size_t hist_bytes(int64_t num) {
   const Plan p = plan(num);
-  return align_up(kBins * sizeof(uint32_t) + (p.fused ? 3 : 1) * table_bytes(p) + 256, 256);
+  return align_up(kBins * sizeof(uint32_t) + table_bytes(p) + 256, 256);
 }
 
-// Counts the digit of every key of a tile.  TILE_MAJOR: hist[tile][digit] and the workgroup also
-// clears its row of `clear` (the table the first scatter launch counts into).
+// Counts the digit of every key of a tile.  TILE_MAJOR: hist[tile][digit], else hist[digit][tile].
 template <typename K, bool TILE_MAJOR>
 __global__ __launch_bounds__(kBlock) void hist_kernel(const K *__restrict__ keys, int64_t num,
                                                       int shift, uint32_t dmask, int rounds,
-                                                      int64_t ntiles, uint32_t *__restrict__ hist,
-                                                      uint32_t *__restrict__ clear) {
+                                                      int64_t ntiles, uint32_t *__restrict__ hist) {
   __shared__ uint32_t h[kBins];
   const int tid = threadIdx.x;
   h[tid] = 0;
@@ -67,7 +65,6 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const K *__restrict__ keys
   __syncthreads();
   if (TILE_MAJOR) {
     hist[(int64_t)blockIdx.x * kBins + tid] = h[tid];
-    clear[(int64_t)blockIdx.x * kBins + tid] = 0u;
   } else {
     hist[(int64_t)tid * ntiles + blockIdx.x] = h[tid];
   }
@@ -101,16 +98,13 @@ __global__ __launch_bounds__(kBlock) void digit_scan_kernel(uint32_t *__restrict
   if (tid == 0) totals[blockIdx.x] = carry;
 }
 
-// FUSED: `table` holds this digit's raw tile-major counts, `next` (may be null on the last digit)
-// receives the counts of the next digit, `clear` (may be null) is zeroed for the launch after.
-// Otherwise `table` holds the digit-major row prefixes and `totals` the digit totals.
+// FUSED: `table` holds this digit's raw tile-major counts.  Otherwise `table` holds the
+// digit-major row prefixes and `totals` the digit totals.
 template <typename K, typename V, bool HAS_V, bool FUSED>
 __global__ __launch_bounds__(kBlock) void scatter_kernel(
     const K *__restrict__ kin, const V *__restrict__ vin, K *__restrict__ kout,
     V *__restrict__ vout, int64_t num, int shift, uint32_t dmask, int rounds, int64_t ntiles,
-    const uint32_t *__restrict__ table, const uint32_t *__restrict__ totals,
-    uint32_t *__restrict__ next, int next_shift, uint32_t next_dmask,
-    uint32_t *__restrict__ clear) {
+    const uint32_t *__restrict__ table, const uint32_t *__restrict__ totals) {
   constexpr int kSub = 4;                  // rounds ranked together: independent ballot chains
   constexpr int kSlots = kSub * kWaves;    // (round, wave) slots of the count table
   __shared__ uint32_t base[kBins];
@@ -170,7 +164,6 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
         before += part[w][0][tid];
         total += part[w][1][tid];
       }
-      if (clear) clear[tile * kBins + tid] = 0u;
     } else {
       before = table[(int64_t)tid * ntiles + tile];
       total = totals[tid];
@@ -186,7 +179,6 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
   }
   __syncthreads();
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  const int64_t tile_elems = (int64_t)kBlock * rounds;
   for (int r0 = 0; r0 < rounds; r0 += kSub) {
     bool valid[kSub];
     uint32_t d[kSub];
@@ -235,10 +227,6 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
         const uint32_t pos = wpre[q * kWaves + wave][d[q]] + (uint32_t)rank[q];
         kout[pos] = kcur[q];
         if (HAS_V) vout[pos] = vcur[q];
-        if (FUSED && next)
-          atomicAdd(&next[(int64_t)(pos / tile_elems) * kBins +
-                          ((uint32_t)(kcur[q] >> next_shift) & next_dmask)],
-                    1u);
       }
     }
     // the next use of wpre is ordered behind this scatter by the barrier after the next ballots
@@ -391,46 +379,32 @@ int sort_pairs(const K *kin, K *kout, const V *vin, V *vout, K *ktmp, V *vtmp, i
   const V *vsrc = vin;
   bool to_out = (passes & 1) != 0;  // alternate so that the last pass writes kout/vout
   uint32_t *totals = hist;
-  uint32_t *tables[3];
-  for (int i = 0; i < 3; ++i) tables[i] = hist + kBins + (p.fused ? i : 0) * (table_bytes(p) / 4);
+  uint32_t *table = hist + kBins;
   const dim3 grid((unsigned)p.ntiles), block(kBlock);
-  auto digit_mask = [&](int shift) {
-    return end_bit - shift >= 8 ? 255u : ((1u << (end_bit - shift)) - 1u);
-  };
-  if (p.fused)
-    hist_kernel<K, true><<<grid, block, 0, st>>>(ksrc, num, begin_bit, digit_mask(begin_bit),
-                                                 p.rounds, p.ntiles, tables[0], tables[1]);
   for (int pass = 0; pass < passes; ++pass) {
     const int shift = begin_bit + 8 * pass;
-    const uint32_t dmask = digit_mask(shift);
+    const uint32_t dmask = end_bit - shift >= 8 ? 255u : ((1u << (end_bit - shift)) - 1u);
     K *kdst = to_out ? kout : ktmp;
     V *vdst = to_out ? vout : vtmp;
     if (p.fused) {
-      const bool last = pass + 1 == passes;
-      uint32_t *next = last ? nullptr : tables[(pass + 1) % 3];
-      uint32_t *clear = pass + 2 < passes ? tables[(pass + 2) % 3] : nullptr;
-      const int nshift = last ? 0 : shift + 8;
-      const uint32_t nmask = last ? 0u : digit_mask(nshift);
+      hist_kernel<K, true><<<grid, block, 0, st>>>(ksrc, num, shift, dmask, p.rounds, p.ntiles,
+                                                   table);
       if (has_v)
         scatter_kernel<K, V, true, true><<<grid, block, 0, st>>>(
-            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, tables[pass % 3],
-            nullptr, next, nshift, nmask, clear);
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, nullptr);
       else
         scatter_kernel<K, V, false, true><<<grid, block, 0, st>>>(
-            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, tables[pass % 3],
-            nullptr, next, nshift, nmask, clear);
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, nullptr);
     } else {
       hist_kernel<K, false><<<grid, block, 0, st>>>(ksrc, num, shift, dmask, p.rounds, p.ntiles,
-                                                    tables[0], nullptr);
-      digit_scan_kernel<<<dim3(kBins), block, 0, st>>>(tables[0], p.ntiles, totals);
+                                                    table);
+      digit_scan_kernel<<<dim3(kBins), block, 0, st>>>(table, p.ntiles, totals);
       if (has_v)
         scatter_kernel<K, V, true, false><<<grid, block, 0, st>>>(
-            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, tables[0], totals,
-            nullptr, 0, 0u, nullptr);
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, totals);
       else
         scatter_kernel<K, V, false, false><<<grid, block, 0, st>>>(
-            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, tables[0], totals,
-            nullptr, 0, 0u, nullptr);
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, totals);
     }
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     ksrc = kdst;
