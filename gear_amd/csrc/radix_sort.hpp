@@ -58,9 +58,18 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const K *__restrict__ keys
   h[tid] = 0;
   __syncthreads();
   const int64_t base = (int64_t)blockIdx.x * kBlock * rounds;
-  for (int r = 0; r < rounds; ++r) {
-    const int64_t i = base + (int64_t)r * kBlock + tid;
-    if (i < num) atomicAdd(&h[(uint32_t)(keys[i] >> shift) & dmask], 1u);
+  for (int r0 = 0; r0 < rounds; r0 += 4) {  // four loads in flight before the first LDS atomic
+    K k[4];
+    bool ok[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int64_t i = base + (int64_t)(r0 + q) * kBlock + tid;
+      ok[q] = r0 + q < rounds && i < num;
+      k[q] = ok[q] ? keys[i] : (K)0;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (ok[q]) atomicAdd(&h[(uint32_t)(k[q] >> shift) & dmask], 1u);
   }
   __syncthreads();
   if (TILE_MAJOR) {
