@@ -238,13 +238,15 @@ constexpr int kMaxRanges = 2048;
 // which the scan launch below finds all aggregates ready (no ticket, no publishing, no polling).
 template <typename In, typename Acc, int VE, int NR>
 __global__ __launch_bounds__(kBlock) void range_sum_kernel(const In *__restrict__ in, int64_t n,
-                                                           uint64_t *__restrict__ aggr) {
+                                                           uint64_t *__restrict__ aggr,
+                                                           int64_t first_range) {
   constexpr int kElems = NR * kBlock * VE;
   constexpr int kWaves = kBlock / kWave;
   typedef typename InVec<In, VE>::type in_vec;
   __shared__ Acc red[kWaves];
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-  const int64_t base = (int64_t)blockIdx.x * kElems;
+  const int64_t range = first_range + blockIdx.x;
+  const int64_t base = range * kElems;
   In raw[NR][VE];
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
@@ -269,13 +271,14 @@ __global__ __launch_bounds__(kBlock) void range_sum_kernel(const In *__restrict_
   const Acc w = wave_sum(tsum);
   if (lane == 0) red[wave] = w;
   __syncthreads();
-  if (tid == 0) aggr[blockIdx.x] = Bits<Acc>::to((red[0] + red[1]) + (red[2] + red[3]));
+  if (tid == 0) aggr[range] = Bits<Acc>::to((red[0] + red[1]) + (red[2] + red[3]));
 }
 
 template <typename In, typename Acc, typename Out, int VE, int NR, bool TWO>
 __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restrict__ in,
                                                              Out *__restrict__ out, int64_t n,
-                                                             uint32_t *ticket, uint64_t *aggr) {
+                                                             uint32_t *ticket, uint64_t *aggr,
+                                                             int64_t first_range) {
   constexpr int kElems = NR * kBlock * VE;
   constexpr int kWaves = kBlock / kWave;
   typedef typename InVec<In, VE>::type in_vec;
@@ -289,7 +292,7 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
     if (tid == 0) s_tile = atomicAdd(ticket, 1u);
     __syncthreads();
   }
-  const int64_t tile = TWO ? (int64_t)blockIdx.x : (int64_t)s_tile;
+  const int64_t tile = TWO ? first_range + (int64_t)blockIdx.x : (int64_t)s_tile;
   const int64_t base = tile * kElems;
 
   In raw[NR][VE];
@@ -428,15 +431,22 @@ size_t scan_ws_bytes(int64_t n) {
   return kHeaderBytes + align_up((size_t)tiles * 16, 256);
 }
 
+// first_changed > 0 (two-launch variant only): the range sums of the ranges before the one that
+// holds element first_changed are still in the workspace from the last scan of this array, and
+// `out` still holds the prefix up to there; only the later ranges are summed and scanned again.
 template <typename In, typename Acc, typename Out, int VE, int NR>
-int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, bool single_pass) {
-  const int64_t ranges = ceil_div64(n, (int64_t)NR * kBlock * VE);
+int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, bool single_pass,
+                  int64_t first_changed) {
+  const int64_t range_elems = (int64_t)NR * kBlock * VE;
+  const int64_t ranges = ceil_div64(n, range_elems);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
   uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
   if (!single_pass) {
-    range_sum_kernel<In, Acc, VE, NR><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(in, n, aggr);
-    scan_ranges_kernel<In, Acc, Out, VE, NR, true><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(
-        in, out, n, ticket, aggr);
+    const int64_t first = first_changed > 0 ? first_changed / range_elems : 0;
+    const dim3 grid((unsigned)(ranges - first)), block(kBlock);
+    range_sum_kernel<In, Acc, VE, NR><<<grid, block, 0, st>>>(in, n, aggr, first);
+    scan_ranges_kernel<In, Acc, Out, VE, NR, true><<<grid, block, 0, st>>>(in, out, n, ticket, aggr,
+                                                                          first);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
@@ -444,13 +454,14 @@ int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, b
                                                                                       ranges);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   scan_ranges_kernel<In, Acc, Out, VE, NR, false><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(
-      in, out, n, ticket, aggr);
+      in, out, n, ticket, aggr, 0);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
 
 template <typename In, typename Acc, typename Out, int VE>
-int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hipStream_t st) {
+int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hipStream_t st,
+                int64_t first_changed = 0) {
   if (n < 0 || n > (1ll << 40)) return n < 0 ? GEAR_HIP_EINVAL : GEAR_HIP_ERANGE;
   if (n == 0) return 0;
   if (!in || !out) return GEAR_HIP_EINVAL;
@@ -467,13 +478,13 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
   const bool single_pass = env_int("GEAR_HIP_SCAN_SINGLE_PASS", 0) != 0;
   const int64_t cap = single_pass ? 1024 : kMaxRanges;
   if (!single_pass && ceil_div64(n, 2 * row) <= cap)
-    return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, single_pass);
+    return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, single_pass, first_changed);
   if (ceil_div64(n, 4 * row) <= cap)
-    return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, single_pass);
+    return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, single_pass, first_changed);
   if (ceil_div64(n, 8 * row) <= cap)
-    return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, single_pass);
+    return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, single_pass, first_changed);
   if (ceil_div64(n, 16 * row) <= kMaxRanges)
-    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, single_pass);
+    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, single_pass, first_changed);
   const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
   uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
@@ -499,6 +510,15 @@ extern "C" int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, vo
                                      size_t workspace_bytes, void *stream) {
   return launch_scan<float, double, double, 4>(in, out, n, workspace, workspace_bytes,
                                                as_stream(stream));
+}
+
+extern "C" int gear_hip_rescan_f32_f64(const float *in, double *out, int64_t n,
+                                       int64_t first_changed, void *workspace,
+                                       size_t workspace_bytes, void *stream) {
+  if (first_changed < 0) return GEAR_HIP_EINVAL;
+  if (first_changed >= n && n >= 0) return 0;  // nothing changed
+  return launch_scan<float, double, double, 4>(in, out, n, workspace, workspace_bytes,
+                                               as_stream(stream), first_changed);
 }
 
 extern "C" int gear_hip_scan_i64(const int64_t *in, int64_t *out, int64_t n, void *workspace,

@@ -88,9 +88,22 @@ class OfflineLoader(BasicLoader):
         """Upload priorities and trajectory lengths after the host side changed them."""
         self._device_weights = self._iset.weights.to(self._mpu.device)
         self._device_timesteps = self._iset.timesteps.to(self._mpu.device)
+        self._dirty_from = 0   # first priority that changed since the sampler last scanned them
+
+    def _mark_dirty(self, local_indices):
+        """Lower the rescan start to the smallest updated index when that is known on the host
+        (a CPU tensor); device-side index tensors would need a synchronisation, so they make
+        the next scan a full one."""
+        if isinstance(local_indices, torch.Tensor) and not local_indices.is_cuda \
+                and local_indices.numel() > 0:
+            self._dirty_from = min(self._dirty_from, max(int(local_indices.min()), 0))
+        else:
+            self._dirty_from = 0
 
     def update_priorities(self, indices, values, unique_indices=False):
         """weights[indices] = values on the device copy (last write wins for duplicates)."""
+        self._mark_dirty(indices - self._iset.index_offset
+                         if isinstance(indices, torch.Tensor) and not indices.is_cuda else None)
         idx = indices.to(self._mpu.device, torch.int64).contiguous()
         if self._iset.index_offset:
             idx = idx - self._iset.index_offset
@@ -115,6 +128,7 @@ class OfflineLoader(BasicLoader):
         ts = self._upd_idx[cap:cap + num]
         w = self._upd_w[:num]
         local = idx - self._iset.index_offset if self._iset.index_offset else idx
+        self._mark_dirty(local)
         self._iset.weights[local] = w
         self._iset.timesteps[local] = ts
         dev = self._mpu.device
@@ -152,7 +166,9 @@ class OfflineLoader(BasicLoader):
 
     def fused_iterate(self):
         sampled = self._sampler.sync_sample(self._indices, self._device_weights,
-                                            self._batch_size * self._dp_world)
+                                            self._batch_size * self._dp_world,
+                                            dirty_from=self._dirty_from)
+        self._dirty_from = self._device_weights.numel()   # clean until the next update
         local = sampled
         if self._iset.index_offset:
             local = sampled - self._iset.index_offset

@@ -205,6 +205,43 @@ def prefix_sum(priorities, out=None):
     return out
 
 
+class PrefixState:
+    """The fp64 prefix of ONE priority array together with a workspace of its own, so that the
+    range sums of the last scan survive other scans and a rescan can start at the first changed
+    priority (gear_hip_rescan_f32_f64).  All calls must be enqueued on the same stream."""
+
+    def __init__(self):
+        self.out = None
+        self._ws = None
+        self._n = -1
+        self._src = None
+        self._valid = False
+
+    def scan(self, priorities, first_changed=0):
+        """first_changed = 0: full scan; k > 0: only priorities[k:] changed since the last call;
+        k >= n: nothing changed (no launch).  Returns the fp64 prefix (the same tensor each call)."""
+        _need(priorities, torch.float32, "priorities")
+        n = priorities.numel()
+        if self.out is None or self._n != n or self.out.device != priorities.device:
+            self.out = torch.empty(n, dtype=torch.float64, device=priorities.device)
+            nbytes = load().gear_hip_scan_workspace_bytes(n)
+            self._ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8,
+                                   device=priorities.device)
+            self._n = n
+            self._valid = False
+        if self._src != priorities.data_ptr():
+            self._valid = False
+        if not self._valid or first_changed <= 0:
+            call("gear_hip_scan_f32_f64", _ptr(priorities), _ptr(self.out), n, _ptr(self._ws),
+                 self._ws.numel(), _stream())
+        else:
+            call("gear_hip_rescan_f32_f64", _ptr(priorities), _ptr(self.out), n,
+                 int(first_changed), _ptr(self._ws), self._ws.numel(), _stream())
+        self._src = priorities.data_ptr()
+        self._valid = True
+        return self.out
+
+
 def prefix_sum_i64(weights, out=None):
     _need(weights, torch.int64, "weights")
     n = weights.numel()

@@ -29,10 +29,15 @@ class UniformSampler:
         self._generator = torch.Generator(mpu.device)
         self._generator.manual_seed(seed)
 
-    def sync_sample(self, indices, weights, batch_size):
+    def sync_sample(self, indices, weights, batch_size, dirty_from=None):
+        """dirty_from (an addition to the reference's signature, used by WeightedSampler): None =
+        the weights may have changed anywhere since the last call; k = only weights[k:] changed;
+        k >= len(weights) = nothing changed."""
         if self._mpu.get_data_parallel_world_size() != 1:
             raise RuntimeError("this build samples on one data-parallel rank only")
-        return self._dp_rank_zero_sync(indices, weights, batch_size)
+        if dirty_from is None:
+            return self._dp_rank_zero_sync(indices, weights, batch_size)
+        return self._dp_rank_zero_sync(indices, weights, batch_size, dirty_from=dirty_from)
 
     def _take_sorted(self, indices, positions):
         """sort(indices[positions]) on the device."""
@@ -40,7 +45,7 @@ class UniformSampler:
         bits = 63
         return ops.sort_i64(picked, key_bits=bits)
 
-    def _dp_rank_zero_sync(self, indices, weights, batch_size):
+    def _dp_rank_zero_sync(self, indices, weights, batch_size, dirty_from=None):
         device = self._mpu.device
         indices = ensure_tensor(indices, device, torch.int64)
         draws = torch.randint(low=0, high=indices.size(0), size=(batch_size,),
@@ -56,15 +61,15 @@ class WeightedSampler(UniformSampler):
     def __init__(self, mpu, seed=42) -> None:
         super().__init__(mpu, seed)
         self._prefix = None
+        self._state = ops.PrefixState()
         self.last_positions = None
 
-    def _dp_rank_zero_sync(self, indices, weights, batch_size):
+    def _dp_rank_zero_sync(self, indices, weights, batch_size, dirty_from=None):
         device = self._mpu.device
         indices = ensure_tensor(indices, device, torch.int64)
         weights = ensure_tensor(weights, device, torch.float32)
-        if self._prefix is None or self._prefix.numel() != weights.numel():
-            self._prefix = torch.empty(weights.numel(), dtype=torch.float64, device=device)
-        ops.prefix_sum(weights, out=self._prefix)
+        # the prefix is rescanned from the first priority that may have changed
+        self._prefix = self._state.scan(weights, 0 if dirty_from is None else int(dirty_from))
         u = torch.rand(batch_size, generator=self._generator, dtype=torch.float32, device=device)
         positions = ops.sample_sorted(self._prefix, u, unit_uniforms=True)
         self.last_positions = positions
@@ -76,9 +81,7 @@ class WeightedSampler(UniformSampler):
         device = self._mpu.device
         indices = ensure_tensor(indices, device, torch.int64)
         weights = ensure_tensor(weights, device, torch.float32)
-        if self._prefix is None or self._prefix.numel() != weights.numel():
-            self._prefix = torch.empty(weights.numel(), dtype=torch.float64, device=device)
-        ops.prefix_sum(weights, out=self._prefix)
+        self._prefix = self._state.scan(weights, 0)
         u = torch.rand(batch_size, generator=self._generator, dtype=torch.float32, device=device)
         positions, is_w = ops.upper_bound(self._prefix, u, unit_uniforms=True, priorities=weights,
                                           beta=beta)
@@ -88,7 +91,7 @@ class WeightedSampler(UniformSampler):
 class TopKSampler(UniformSampler):
     """The batch_size largest priorities (ties: smaller index first), returned as sorted indices."""
 
-    def _dp_rank_zero_sync(self, indices, weights, batch_size):
+    def _dp_rank_zero_sync(self, indices, weights, batch_size, dirty_from=None):
         device = self._mpu.device
         indices = ensure_tensor(indices, device, torch.int64)
         weights = ensure_tensor(weights, device, torch.float32)

@@ -177,7 +177,8 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
 
 /* Inclusive prefix sum of fp32 priorities accumulated and written in fp64:
  *     out[i] = sum_{j<=i} (double) in[j]
- * Single-pass decoupled look-back scan.  Replaces gear::cuda::launch_prefix_sum /
+ * Two-launch range scan (or the single-pass kernels, see GEAR_HIP_SCAN_SINGLE_PASS).  Replaces
+ * gear::cuda::launch_prefix_sum /
  * one_dimension_prefix_sum (src/cuda/one_dim_prefix_sum.cu:125-273; libgear.core.prefix_sum,
  * :276-278), which is fp32 and only correct for one block.
  * workspace: device memory of at least gear_hip_scan_workspace_bytes(n) bytes, 256-byte aligned;
@@ -186,6 +187,18 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
 size_t gear_hip_scan_workspace_bytes(int64_t n);
 int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspace,
                           size_t workspace_bytes, void *stream);
+
+/* Incremental form for the online priority path (priorities of a few trajectories change between
+ * batches: SharedMemoryIndexServer::update, src/index/server.cc:175-180, and
+ * WeightUpdateRequestArray, src/index/request.cc:41-75; the reference has no prefix to maintain).
+ * Preconditions: the last call on (in, out, workspace) was gear_hip_scan_f32_f64 or this function
+ * with the same n, and since then only in[first_changed .. n) changed.  Then out[i] is
+ * recomputed from the start of the range that holds first_changed onwards, reusing the range sums
+ * kept in the workspace; the result is bit-identical to a full gear_hip_scan_f32_f64.
+ * first_changed >= n: nothing to do; first_changed = 0, n > 33.5 M or
+ * GEAR_HIP_SCAN_SINGLE_PASS=1: a full scan. */
+int gear_hip_rescan_f32_f64(const float *in, double *out, int64_t n, int64_t first_changed,
+                            void *workspace, size_t workspace_bytes, void *stream);
 
 /* The same scan (fp64 accumulation) with the result rounded to fp32 on output: the signature of
  * the reference's binding, prefix_sum(FloatTensor input, FloatTensor output)

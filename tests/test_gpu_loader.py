@@ -266,3 +266,33 @@ def test_cached_weight_updates_reach_the_device(oracle):
     val = torch.tensor([1, 2, 3, 4, 5, 6], device="cuda")
     ops.scatter(tab, idx, val, unique_indices=False)
     assert tab[5].item() == 6 and tab[7].item() == 5 and tab[99].item() == 4
+
+
+def test_weighted_loader_rescans_from_the_first_updated_priority(oracle):
+    """Online path with the weighted sampler: after priority updates whose indices are known on the
+    host, the next batch rescans the prefix from the smallest updated index only; the prefix it
+    samples from must equal a full scan of the updated priorities bit for bit, and a batch without
+    updates in between must not change it."""
+    from gear_amd import ops
+    from gear_amd.loader import OfflineLoader
+    ds, raw = _dataset("pinned", seed=11)
+    loader = OfflineLoader(ds, 8, _mpu(), "Weighted", PATTERNS)
+    next(loader)
+    w = ds.weights.numpy().copy()
+    rng = np.random.default_rng(11)
+    for rnd in range(4):
+        idx = torch.from_numpy(rng.integers(5 * rnd + 3, 48, size=6))
+        val = torch.from_numpy(rng.random(6).astype(np.float32) + 0.5)
+        announce("weighted loader update round %d" % rnd)
+        loader.update_priorities(idx, val)
+        oracle.scatter_f32(w, idx.numpy(), val.numpy())
+        assert loader._dirty_from == int(idx.min())
+        timesteps, _ = next(loader)
+        torch.cuda.synchronize()
+        assert loader._dirty_from == 48
+        full = ops.prefix_sum(loader._device_weights)
+        assert torch.equal(loader._sampler._prefix, full)
+        assert np.array_equal(loader._device_weights.cpu().numpy(), w)
+        next(loader)                                   # nothing changed: no rescan, same prefix
+        torch.cuda.synchronize()
+        assert torch.equal(loader._sampler._prefix, full)

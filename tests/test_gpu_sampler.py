@@ -256,3 +256,48 @@ def test_sample_sorted_with_many_equal_indices(oracle, num):
     assert np.array_equal(idxs.cpu().numpy(), exp // T)
     assert np.array_equal(tss.cpu().numpy(), exp % T)
     assert np.array_equal(lens.cpu().numpy(), exp % T + 1)
+
+
+@pytest.mark.parametrize("n", [5_000, 1_000_000, 10_000_003])
+def test_rescan_from_first_changed_is_bit_identical(oracle, n):
+    """gear_hip_rescan_f32_f64: after priorities[k:] changed, rescanning from k gives exactly the
+    bits of a full scan of the changed array (the range sums before k are reused from the
+    workspace), for k inside the first range, on range boundaries, at the end and beyond it."""
+    from gear_amd import ops
+    rng = np.random.default_rng(n)
+    p = _priorities(n, 11)
+    dp = _dev(p)
+    state = ops.PrefixState()
+    state.scan(dp)
+    other = _dev(_priorities(70_000, 12))
+    for k in (1, 2047, 2048, 4096, n // 3, n // 2 + 1, n - 1, n, n + 5):
+        if k < n:
+            m = min(n - k, 1000)
+            pos = k + rng.integers(0, n - k, size=m)
+            pos[0] = k
+            p[pos] = (rng.lognormal(0, 1, size=m) ** 0.6).astype(np.float32)
+            dp.copy_(torch.from_numpy(p))
+        ops.prefix_sum(other)                      # scans of other arrays do not disturb the state
+        announce("rescan n=%d first_changed=%d" % (n, k))
+        got = state.scan(dp, first_changed=k)
+        full = ops.prefix_sum(dp)
+        torch.cuda.synchronize()
+        assert torch.equal(got, full), "first_changed=%d" % k
+    exp = oracle.scan_f32_f64(p)
+    assert np.max(np.abs(got.cpu().numpy() - exp) / exp) <= 1e-12
+
+
+def test_rescan_integer_valued_matches_oracle_exactly(oracle):
+    from gear_amd import ops
+    n = 3_000_017
+    rng = np.random.default_rng(8)
+    p = rng.integers(0, 100, size=n).astype(np.float32)
+    dp = _dev(p)
+    state = ops.PrefixState()
+    state.scan(dp)
+    for k in (2_999_000, 1_500_000, 77):
+        p[k:k + 500] = rng.integers(0, 100, size=500).astype(np.float32)
+        dp.copy_(torch.from_numpy(p))
+        announce("integer rescan first_changed=%d" % k)
+        got = state.scan(dp, first_changed=k).cpu().numpy()
+        assert np.array_equal(got, oracle.scan_f32_f64(p))
