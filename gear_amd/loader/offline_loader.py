@@ -53,7 +53,8 @@ class OfflineLoader(BasicLoader):
 
     def __init__(self, dataset, batch_size: int, mpu, sampling_method: str = "Uniform",
                  patterns: Sequence[Dict[str, Any]] = None, logger: logging.Logger = None,
-                 timesteps_on_device: bool = False, with_mask: bool = False) -> None:
+                 timesteps_on_device: bool = False, with_mask: bool = False,
+                 use_graph: bool = False) -> None:
         super().__init__(batch_size)
         self._dataset = ensure_dataset(dataset)
         self._handler = self._dataset._handler
@@ -74,6 +75,16 @@ class OfflineLoader(BasicLoader):
         self._batch_size = batch_size
         self._timesteps_on_device = timesteps_on_device
         self._with_mask = with_mask
+        # use_graph: select + length look-up + gather are captured once into a HIP graph and
+        # replayed per batch (small batches are bound by host launches, not by the kernels).
+        # The returned tensors are then the SAME buffers every iteration, and the timesteps stay
+        # on the device.
+        self._use_graph = use_graph
+        self._graph = None
+        self._graph_draws = None
+        self._graph_out = None
+        if use_graph and not timesteps_on_device:
+            raise ValueError("use_graph=True needs timesteps_on_device=True (no host copy per batch)")
         self._logger = logger or logging.Logger(name="OfflineLoader", level=logging.DEBUG)
 
         self.refresh_index()
@@ -89,6 +100,7 @@ class OfflineLoader(BasicLoader):
         self._device_weights = self._iset.weights.to(self._mpu.device)
         self._device_timesteps = self._iset.timesteps.to(self._mpu.device)
         self._dirty_from = 0   # first priority that changed since the sampler last scanned them
+        self._graph = None     # a captured step holds the replaced tensors
 
     def _mark_dirty(self, local_indices):
         """Lower the rescan start to the smallest updated index when that is known on the host
@@ -164,7 +176,39 @@ class OfflineLoader(BasicLoader):
         self.last_masks = masks
         return data_batch
 
+    def _graph_step(self):
+        sampled = self._sampler.select(self._indices, self._device_weights, self._graph_draws)
+        local = sampled - self._iset.index_offset if self._iset.index_offset else sampled
+        lengths = ops.take_i64(self._device_timesteps, local)
+        return lengths, self._gather(local, lengths)
+
+    def _graph_iterate(self):
+        n = self._indices.numel()
+        bsz = self._batch_size * self._dp_world
+        draws = self._sampler.draw(n, bsz)          # eager: the random stream stays torch's
+        if self._graph is None:
+            self._graph_draws = draws.clone()
+            side = torch.cuda.Stream(self._mpu.device)
+            side.wait_stream(torch.cuda.current_stream(self._mpu.device))
+            with torch.cuda.stream(side):           # warm-up: workspaces get allocated
+                self._graph_step()
+            torch.cuda.current_stream(self._mpu.device).wait_stream(side)
+            torch.cuda.synchronize(self._mpu.device)
+            self._graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self._graph, stream=side):
+                self._graph_out = self._graph_step()
+        else:
+            self._graph_draws.copy_(draws)
+        self._graph.replay()
+        return self._graph_out
+
+    def refresh_graph(self):
+        """Drop the captured step (after refresh_index or anything else that replaces tensors)."""
+        self._graph = None
+
     def fused_iterate(self):
+        if self._use_graph:
+            return self._graph_iterate()
         sampled = self._sampler.sync_sample(self._indices, self._device_weights,
                                             self._batch_size * self._dp_world,
                                             dirty_from=self._dirty_from)

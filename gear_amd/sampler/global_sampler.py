@@ -24,6 +24,8 @@ def ensure_tensor(v, device, dtype=None):
 
 
 class UniformSampler:
+    _uses_weights = False
+
     def __init__(self, mpu, seed=42) -> None:
         self._mpu = mpu
         self._generator = torch.Generator(mpu.device)
@@ -45,18 +47,31 @@ class UniformSampler:
         bits = 63
         return ops.sort_i64(picked, key_bits=bits)
 
+    # Every sampler is split into draw() -- the random numbers, produced by torch -- and
+    # select() -- everything after them, deterministic and free of host synchronisation, so a
+    # loader can capture select() + gather in a HIP graph and feed it fresh draws.
+    def draw(self, num_indices, batch_size):
+        return torch.randint(low=0, high=num_indices, size=(batch_size,),
+                             generator=self._generator, dtype=torch.long,
+                             device=self._mpu.device)
+
+    def select(self, indices, weights, draws, dirty_from=None):
+        return self._take_sorted(indices, draws)
+
     def _dp_rank_zero_sync(self, indices, weights, batch_size, dirty_from=None):
         device = self._mpu.device
         indices = ensure_tensor(indices, device, torch.int64)
-        draws = torch.randint(low=0, high=indices.size(0), size=(batch_size,),
-                              generator=self._generator, dtype=torch.long, device=device)
-        return self._take_sorted(indices, draws)
+        if self._uses_weights:
+            weights = ensure_tensor(weights, device, torch.float32)
+        return self.select(indices, weights, self.draw(indices.size(0), batch_size),
+                           dirty_from=dirty_from)
 
 
 class WeightedSampler(UniformSampler):
     """Priority-proportional sampling with replacement: inclusive fp64 prefix sum of the
     priorities, then upper_bound of seeded uniforms in [0, sum).  Entries with priority 0 are
     never drawn."""
+    _uses_weights = True
 
     def __init__(self, mpu, seed=42) -> None:
         super().__init__(mpu, seed)
@@ -64,14 +79,14 @@ class WeightedSampler(UniformSampler):
         self._state = ops.PrefixState()
         self.last_positions = None
 
-    def _dp_rank_zero_sync(self, indices, weights, batch_size, dirty_from=None):
-        device = self._mpu.device
-        indices = ensure_tensor(indices, device, torch.int64)
-        weights = ensure_tensor(weights, device, torch.float32)
+    def draw(self, num_indices, batch_size):
+        return torch.rand(batch_size, generator=self._generator, dtype=torch.float32,
+                          device=self._mpu.device)
+
+    def select(self, indices, weights, draws, dirty_from=None):
         # the prefix is rescanned from the first priority that may have changed
         self._prefix = self._state.scan(weights, 0 if dirty_from is None else int(dirty_from))
-        u = torch.rand(batch_size, generator=self._generator, dtype=torch.float32, device=device)
-        positions = ops.sample_sorted(self._prefix, u, unit_uniforms=True)
+        positions = ops.sample_sorted(self._prefix, draws, unit_uniforms=True)
         self.last_positions = positions
         return self._take_sorted(indices, positions)
 
@@ -90,10 +105,11 @@ class WeightedSampler(UniformSampler):
 
 class TopKSampler(UniformSampler):
     """The batch_size largest priorities (ties: smaller index first), returned as sorted indices."""
+    _uses_weights = True
 
-    def _dp_rank_zero_sync(self, indices, weights, batch_size, dirty_from=None):
-        device = self._mpu.device
-        indices = ensure_tensor(indices, device, torch.int64)
-        weights = ensure_tensor(weights, device, torch.float32)
-        _, positions = ops.topk(weights, batch_size, sorted_by_value=False, want_values=False)
+    def draw(self, num_indices, batch_size):
+        return torch.empty(batch_size, dtype=torch.int64, device=self._mpu.device)  # size only
+
+    def select(self, indices, weights, draws, dirty_from=None):
+        _, positions = ops.topk(weights, draws.numel(), sorted_by_value=False, want_values=False)
         return self._take_sorted(indices, positions)

@@ -296,3 +296,30 @@ def test_weighted_loader_rescans_from_the_first_updated_priority(oracle):
         next(loader)                                   # nothing changed: no rescan, same prefix
         torch.cuda.synchronize()
         assert torch.equal(loader._sampler._prefix, full)
+
+
+@pytest.mark.parametrize("method", ["Uniform", "Weighted", "Topk"])
+def test_graph_loader_equals_eager_loader(method):
+    """use_graph=True captures select + length look-up + gather once and replays it per batch;
+    with the same seed every batch must equal the eager loader's, also after a priority update."""
+    from gear_amd.loader import OfflineLoader
+    name = {"Topk": "TopK"}.get(method, method)
+    ds, raw = _dataset("device", seed=21)
+    eager = OfflineLoader(ds, 16, _mpu(), name, PATTERNS, timesteps_on_device=True)
+    graph = OfflineLoader(ds, 16, _mpu(), name, PATTERNS, timesteps_on_device=True,
+                          use_graph=True)
+    with pytest.raises(ValueError):
+        OfflineLoader(ds, 16, _mpu(), name, PATTERNS, use_graph=True)
+    for it in range(6):
+        if it == 3:
+            idx = torch.tensor([1, 17, 30, 44])
+            val = torch.tensor([50.0, 40.0, 30.0, 20.0])
+            eager.update_priorities(idx, val)
+            graph.update_priorities(idx, val)
+        announce("graph loader %s iteration %d" % (method, it))
+        ts_e, b_e = next(eager)
+        ts_g, b_g = next(graph)
+        torch.cuda.synchronize()
+        assert torch.equal(ts_e, ts_g), "iteration %d" % it
+        for a, b in zip(b_e, b_g):
+            assert torch.equal(a, b), "iteration %d" % it
