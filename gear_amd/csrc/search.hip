@@ -1,8 +1,10 @@
-// Batched upper_bound of draws in an inclusive prefix array (+ importance weights), gfx950.
+// Batched upper_bound of draws in an inclusive prefix array (+ importance weights), and the
+// one-call batch sampler (search + ranking sort + split into window arguments), gfx950.
 //
-// One thread per draw.  The first levels of the binary search touch the same few prefix entries
-// for every draw, so they are served by the caches; the search is latency-bound
-// (log2(n) dependent loads), which is why all draws of a batch run concurrently.
+// One thread per draw, one wave per workgroup.  The first levels of the search touch the same few
+// prefix entries for every draw, so they are served by the caches; the search is latency-bound
+// (a chain of log8(n) + 1 dependent load steps), which is why all draws of a batch run concurrently
+// and spread over many CUs.
 #include <math.h>
 
 #include "radix_sort.hpp"
