@@ -21,7 +21,8 @@ constexpr int kMaxHistBlocks = 512;
 struct State {
   uint32_t prefix[3];  // key bits decided after pass 0, 1, 2 (right-aligned)
   uint32_t k_rem[3];   // entries still to take from the bin picked in that pass
-  uint32_t pad[58];
+  uint32_t overflow;   // a wave found more candidates than its list holds: the write launch re-reads
+  uint32_t pad[57];
 };
 static_assert(sizeof(State) == 256, "State is the 256-byte header of the workspace");
 
@@ -31,16 +32,48 @@ __device__ __forceinline__ uint32_t order_key(float f) {
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 
+constexpr int kStep = kWave * 4;  // elements one wave handles per step (one float4 per lane)
+constexpr int kAhead = 4;         // steps whose loads are in flight together
+
+// Geometry of the compaction launches: `ranges` workgroups, every wave owns wave_len consecutive
+// elements (a multiple of kStep) and a candidate list of list_cap entries.
+struct Geom {
+  int64_t ranges, wave_len, list_cap;
+};
+
+Geom geom(int64_t n, int64_t k) {
+  Geom g;
+  g.ranges = ceil_div64(n > 0 ? n : 1, (int64_t)kWavesPerBlock * kAhead * kStep);
+  if (g.ranges > kMaxRanges) g.ranges = kMaxRanges;
+  g.wave_len = ceil_div64(ceil_div64(n > 0 ? n : 1, g.ranges * kWavesPerBlock), kStep) * kStep;
+  g.ranges = ceil_div64(n > 0 ? n : 1, g.wave_len * kWavesPerBlock);
+  // four times a wave's fair share of the k selected entries, at least 64, never more than the
+  // wave has elements; clustered maxima or many ties overflow it and take the re-reading path
+  const int64_t waves = g.ranges * kWavesPerBlock;
+  int64_t cap = ceil_div64(4 * ceil_div64(k > 0 ? k : 1, waves), 64) * 64;
+  if (cap < 64) cap = 64;
+  if (cap > g.wave_len) cap = g.wave_len;
+  g.list_cap = cap;
+  return g;
+}
+
+// the priority whose order_key is `key` (for +-0.0: +0.0)
+__device__ __forceinline__ float key_to_float(uint32_t key) {
+  return __uint_as_float((key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
+}
+
 struct Layout {
-  size_t hist, desc, ckey, cidx, skey, sidx, tkey, tidx, shist, total;
+  size_t hist, desc, lists, ckey, cidx, skey, sidx, tkey, tidx, shist, total;
 };
 
 Layout layout(int64_t n, int64_t k) {
   Layout l;
   const size_t kk = align_up((size_t)(k > 0 ? k : 1) * 4, 256);
+  const Geom g = geom(n, k);
   size_t o = sizeof(State);
   l.hist = o;  o += 3 * kHistBins * sizeof(uint32_t);
   l.desc = o;  o += (size_t)kMaxRanges * (kWavesPerBlock + 1) * 8;  // wave and workgroup counts
+  l.lists = o; o += align_up((size_t)(g.ranges * kWavesPerBlock * g.list_cap) * 4, 256);
   l.ckey = o;  o += kk;
   l.cidx = o;  o += kk;
   l.skey = o;  o += kk;
@@ -123,14 +156,21 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__rest
   if (PASS == 2) prefix = pick_bin<1>(k, state, hist - kHistBins).prefix;
   __syncthreads();
 
+  // Passes 1 and 2 count only the keys that start with `prefix`: about 1 % of the input.  Whether
+  // a priority is one of them is decided with two float compares against the bounds of that key
+  // range (float order = key order for non-NaN values, -0.0 == +0.0); the key itself is worked
+  // out only for the members.
+  constexpr int kLowBits = PASS == 1 ? 21 : 10;
+  const uint32_t lo_key = PASS == 0 ? 0u : prefix << kLowBits;
+  uint32_t hi_key = PASS == 0 ? 0u : (lo_key | ((1u << kLowBits) - 1u));
+  if (hi_key == 0x7fffffffu) hi_key = 0x7ffffffeu;  // the key below +-0.0's: the zeros are not in this range
+  const float lo_f = key_to_float(lo_key), hi_f = key_to_float(hi_key);
   auto count = [&](float f) {
-    const uint32_t key = order_key(f);
     if (PASS == 0) {
-      atomicAdd(&h[key >> 21], 1u);
-    } else if (PASS == 1) {
-      if ((key >> 21) == prefix) atomicAdd(&h[(key >> 10) & 0x7ffu], 1u);
-    } else {
-      if ((key >> 10) == prefix) atomicAdd(&h[key & 0x3ffu], 1u);
+      atomicAdd(&h[order_key(f) >> 21], 1u);
+    } else if (f >= lo_f && f <= hi_f) {
+      const uint32_t key = order_key(f);
+      atomicAdd(&h[PASS == 1 ? ((key >> 10) & 0x7ffu) : (key & 0x3ffu)], 1u);
     }
   };
   const int64_t nvec = n >> 2;
@@ -165,9 +205,6 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__rest
 // launch writes every wave's packed (greater << 31 | equal) count and every workgroup's total; the
 // write launch sums the totals of the workgroups before it, adds the counts of the waves before it
 // in its own workgroup, and walks its range again (now from L2 / MALL) placing the selected entries.
-constexpr int kStep = kWave * 4;  // elements one wave handles per step (one float4 per lane)
-constexpr int kAhead = 4;         // steps whose loads are in flight together
-
 typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
 
 __device__ __forceinline__ void load_quad(const float *__restrict__ p, int64_t e0, int64_t end,
@@ -183,36 +220,75 @@ __device__ __forceinline__ void load_quad(const float *__restrict__ p, int64_t e
 
 __global__ __launch_bounds__(kBlock) void count_ranges_kernel(
     const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist2,
-    int64_t wave_len, uint64_t *__restrict__ wave_counts, uint64_t *__restrict__ block_counts) {
+    int64_t wave_len, uint64_t *__restrict__ wave_counts, uint64_t *__restrict__ block_counts,
+    uint32_t *__restrict__ lists, int list_cap) {
   __shared__ int64_t red[kWavesPerBlock];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   const int64_t begin = gw * wave_len;
   const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+  uint32_t *list = lists + gw * list_cap;
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  int listed = 0;         // candidates of this wave so far (wave-uniform)
+  bool overflow = false;  // wave-uniform
   // the first loads are issued before the threshold is picked so that the two latencies overlap
   float q[kAhead][4];
 #pragma unroll
   for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
-  const uint32_t thr = pick_bin<2>(k, state, hist2).prefix;
+  const float thr_f = key_to_float(pick_bin<2>(k, state, hist2).prefix);
   uint32_t gt = 0, eq = 0;
   for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
-    if (s0 != begin) {
+    // the next batch of loads is in flight while this one is classified and listed
+    float qn[kAhead][4];
+    const int64_t s1 = s0 + kAhead * kStep;
+    if (s1 < end) {
 #pragma unroll
-      for (int a = 0; a < kAhead; ++a) load_quad(p, s0 + (int64_t)a * kStep + lane * 4, end, q[a]);
+      for (int a = 0; a < kAhead; ++a) load_quad(p, s1 + (int64_t)a * kStep + lane * 4, end, qn[a]);
     }
 #pragma unroll
     for (int a = 0; a < kAhead; ++a) {
       const int64_t e0 = s0 + (int64_t)a * kStep + lane * 4;
+      // every candidate (greater than, or equal to, the threshold) goes to the wave's list in
+      // index order as index | greater << 31; the write launch then never reads the priorities
+      bool sel[4];
+      uint32_t val[4];
+      int off[4], nc = 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t key = order_key(q[a][j]);
-        if (e0 + j < end) {
-          gt += key > thr;
-          eq += key == thr;
-        }
+        // float compares order non-NaN priorities exactly like their keys (-0.0 == +0.0) at
+        // one instruction each
+        const bool above = q[a][j] > thr_f;
+        sel[j] = e0 + j < end && q[a][j] >= thr_f;
+        off[j] = nc;
+        nc += sel[j] ? 1 : 0;
+        gt += sel[j] && above;
+        eq += sel[j] && !above;
+        val[j] = (uint32_t)(e0 + j) | (above ? 0x80000000u : 0u);
       }
+      if (wave_ballot(nc != 0) == 0ull) continue;
+      // candidates in the lanes before this one: nc <= 4 is three bits, one ballot per bit
+      // (independent instructions; a DPP scan is a chain of a dozen dependent ones)
+      const uint64_t b0 = wave_ballot((nc & 1) != 0), b1 = wave_ballot((nc & 2) != 0),
+                     b2 = wave_ballot((nc & 4) != 0);
+      const int before = __popcll(b0 & lt_mask) + 2 * __popcll(b1 & lt_mask) +
+                         4 * __popcll(b2 & lt_mask);
+      const int total = __popcll(b0) + 2 * __popcll(b1) + 4 * __popcll(b2);
+      if (listed + total > list_cap) {
+        overflow = true;
+      } else {
+        const int at = listed + before;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (sel[j]) list[at + off[j]] = val[j];
+      }
+      listed += total;
     }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q[a][j] = qn[a][j];
   }
+  if (overflow && lane == 0) state->overflow = 1u;  // same value from every overflowing wave
   const int64_t w = wave_sum(((int64_t)gt << 31) | (int64_t)eq);
   if (lane == 0) {
     wave_counts[gw] = (uint64_t)w;
@@ -231,17 +307,21 @@ template <bool DIRECT>
 __global__ __launch_bounds__(kBlock) void write_ranges_kernel(
     const float *__restrict__ p, int64_t n, const State *state, int64_t wave_len,
     const uint64_t *__restrict__ wave_counts, const uint64_t *__restrict__ block_counts,
-    uint32_t *__restrict__ ckey, uint32_t *__restrict__ cidx, float *__restrict__ values_out,
+    const uint32_t *__restrict__ lists, int list_cap, uint32_t *__restrict__ ckey,
+    uint32_t *__restrict__ cidx, float *__restrict__ values_out,
     int64_t *__restrict__ indices_out) {
   __shared__ int64_t red[kWavesPerBlock];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   const int64_t begin = gw * wave_len;
   const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+  const bool reread = state->overflow != 0u;  // some wave's list was too short: all waves re-read
   float q[kAhead][4];
+  if (reread) {
 #pragma unroll
-  for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
-  const uint32_t thr = state->prefix[2];
+    for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
+  }
+  const float thr_f = key_to_float(state->prefix[2]);
   const uint32_t need_eq = state->k_rem[2];
 
   int64_t part = 0;
@@ -258,6 +338,40 @@ __global__ __launch_bounds__(kBlock) void write_ranges_kernel(
   excl += wave_sum(own);
   uint32_t gt_run = (uint32_t)(excl >> 31), eq_run = (uint32_t)(excl & 0x7fffffff);
 
+  auto emit = [&](uint32_t pos, int64_t index, float value, uint32_t key) {
+    if (DIRECT) {
+      indices_out[pos] = index;
+      if (values_out) values_out[pos] = value;
+    } else {
+      ckey[pos] = ~key;
+      cidx[pos] = (uint32_t)index;
+    }
+  };
+
+  if (!reread) {
+    // the wave's candidates, in index order, from its list
+    const uint64_t mine = wave_counts[gw];
+    const int m = (int)(mine >> 31) + (int)(mine & 0x7fffffff);
+    const uint32_t *list = lists + gw * list_cap;
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    for (int c0 = 0; c0 < m; c0 += kWave) {
+      const bool valid = c0 + lane < m;
+      const uint32_t ent = valid ? list[c0 + lane] : 0u;
+      const bool is_gt = valid && (ent >> 31) != 0u, is_eq = valid && (ent >> 31) == 0u;
+      const uint64_t bg = wave_ballot(is_gt), be = wave_ballot(is_eq);
+      const uint32_t g = gt_run + (uint32_t)__popcll(bg & lt_mask);
+      const uint32_t e = eq_run + (uint32_t)__popcll(be & lt_mask);
+      if (is_gt || (is_eq && e < need_eq)) {
+        const uint32_t index = ent & 0x7fffffffu;
+        const float value = p[index];
+        emit(g + (e < need_eq ? e : need_eq), (int64_t)index, value, order_key(value));
+      }
+      gt_run += (uint32_t)__popcll(bg);
+      eq_run += (uint32_t)__popcll(be);
+    }
+    return;
+  }
+
   for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
     if (s0 != begin) {
 #pragma unroll
@@ -266,13 +380,10 @@ __global__ __launch_bounds__(kBlock) void write_ranges_kernel(
 #pragma unroll
     for (int a = 0; a < kAhead; ++a) {
       const int64_t e0 = s0 + (int64_t)a * kStep + lane * 4;
-      uint32_t key[4];
       int s = 0;  // packed counts of the lane's four entries: greater << 16 | equal
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        key[j] = order_key(q[a][j]);
-        if (e0 + j < end) s += key[j] > thr ? (1 << 16) : (key[j] == thr ? 1 : 0);
-      }
+      for (int j = 0; j < 4; ++j)
+        if (e0 + j < end) s += q[a][j] > thr_f ? (1 << 16) : (q[a][j] == thr_f ? 1 : 0);
       if (wave_ballot(s != 0) == 0ull) continue;
       const int inc = wave_inclusive_sum(s);
       const int total = wave_read_lane(inc, kWave - 1);
@@ -282,17 +393,9 @@ __global__ __launch_bounds__(kBlock) void write_ranges_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (e0 + j < end) {
-          const bool is_gt = key[j] > thr, is_eq = key[j] == thr;
-          if (is_gt || (is_eq && e < need_eq)) {
-            const uint32_t pos = g + (e < need_eq ? e : need_eq);
-            if (DIRECT) {
-              indices_out[pos] = e0 + j;
-              if (values_out) values_out[pos] = q[a][j];
-            } else {
-              ckey[pos] = ~key[j];
-              cidx[pos] = (uint32_t)(e0 + j);
-            }
-          }
+          const bool is_gt = q[a][j] > thr_f, is_eq = q[a][j] == thr_f;
+          if (is_gt || (is_eq && e < need_eq))
+            emit(g + (e < need_eq ? e : need_eq), e0 + j, q[a][j], order_key(q[a][j]));
           g += is_gt;
           e += is_eq;
         }
@@ -353,23 +456,24 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   uint32_t *ckey = reinterpret_cast<uint32_t *>(ws + l.ckey);
   uint32_t *cidx = reinterpret_cast<uint32_t *>(ws + l.cidx);
   const bool direct = !sorted_by_value;
-  int64_t ranges = ceil_div64(n, (int64_t)kWavesPerBlock * kAhead * kStep);
-  if (ranges > kMaxRanges) ranges = kMaxRanges;
-  const int64_t wave_len = ceil_div64(ceil_div64(n, ranges * kWavesPerBlock), kStep) * kStep;
-  ranges = ceil_div64(n, wave_len * kWavesPerBlock);
+  const Geom g = geom(n, k);
+  const int64_t ranges = g.ranges, wave_len = g.wave_len;
+  uint32_t *lists = reinterpret_cast<uint32_t *>(ws + l.lists);
   uint64_t *wave_counts = reinterpret_cast<uint64_t *>(ws + l.desc);
   uint64_t *block_counts = wave_counts + (size_t)kMaxRanges * kWavesPerBlock;
   const dim3 cgrid((unsigned)ranges);
   count_ranges_kernel<<<cgrid, block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins,
-                                               wave_len, wave_counts, block_counts);
+                                               wave_len, wave_counts, block_counts, lists,
+                                               (int)g.list_cap);
   if (direct)
     write_ranges_kernel<true><<<cgrid, block, 0, st>>>(priorities, n, state, wave_len, wave_counts,
-                                                       block_counts, ckey, cidx, values_out,
-                                                       indices_out);
+                                                       block_counts, lists, (int)g.list_cap, ckey,
+                                                       cidx, values_out, indices_out);
   else
     write_ranges_kernel<false><<<cgrid, block, 0, st>>>(priorities, n, state, wave_len,
-                                                        wave_counts, block_counts, ckey, cidx,
-                                                        values_out, indices_out);
+                                                        wave_counts, block_counts, lists,
+                                                        (int)g.list_cap, ckey, cidx, values_out,
+                                                        indices_out);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   if (direct) return 0;
   uint32_t *skey = reinterpret_cast<uint32_t *>(ws + l.skey);

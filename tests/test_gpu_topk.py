@@ -47,6 +47,14 @@ def test_topk_cases(oracle):
     _check_topk(oracle, ops, special, 19_998, "zeros / inf / denormals")
     mixed = rng.normal(size=50_000).astype(np.float32)  # negative values order correctly too
     _check_topk(oracle, ops, mixed, 12_345, "signed")
+    # clustered maxima: every selected entry sits in a few waves, whose candidate lists overflow,
+    # so the write launch takes its re-reading path; ascending, descending, and one hot block
+    _check_topk(oracle, ops, np.sort(ln(300_000)), 5_000, "ascending (lists overflow)")
+    _check_topk(oracle, ops, np.sort(ln(300_000))[::-1].copy(), 5_000, "descending (lists overflow)")
+    hot = ln(2_000_000)
+    hot[777_000:780_000] += 1000.0
+    _check_topk(oracle, ops, hot, 2_500, "one hot stretch (lists overflow)")
+    _check_topk(oracle, ops, ln(2_000_000), 2_500, "same size, spread out (lists)")
 
 
 def test_topk_config5_size(oracle):
