@@ -1,12 +1,16 @@
 // Top-k of fp32 priorities by radix select + ordered compaction + radix sort, gfx950.
 //
 // fp32 priorities map to order-preserving uint32 keys.  Three histogram passes (11 + 11 + 10
-// bits, LDS histograms, the consuming launch picks the bin) find the key T of the k-th
-// largest priority and how many entries equal to T are still needed.  An ordered compaction (a
-// count launch and a write launch over packed (greater, equal) counts) writes the selected entries
-// in index order: every entry above T, and the first need_eq entries equal to T -- ties go to the
-// smaller index.  For value order the k candidates then go through the stable LSD radix sort on the
-// inverted key.
+// bits, LDS histograms, the consuming launch picks the bin) find the key T of the k-th largest
+// priority and how many entries equal to T are still needed.  An ordered compaction in two
+// launches writes the selected entries in index order: every entry above T, and the first need_eq
+// entries equal to T -- ties go to the smaller index.  The count launch also lists every wave's
+// candidates (entries >= T), so the write launch touches only those; where the maxima are
+// clustered a list overflows and the write launch re-reads the priorities instead.  For value
+// order the k candidates then go through the stable LSD radix sort on the inverted key.
+// The streaming loops are sensitive to their instruction count (a launch that reads 40 MB spends
+// as long issuing ~10 instructions per element as waiting for memory), so they compare floats
+// (one instruction, same order as the keys for non-NaN values) wherever a key is not needed.
 #include "radix_sort.hpp"
 
 namespace gearhip {
@@ -27,9 +31,11 @@ struct State {
 static_assert(sizeof(State) == 256, "State is the 256-byte header of the workspace");
 
 __device__ __forceinline__ uint32_t order_key(float f) {
-  uint32_t b = __float_as_uint(f);
-  if (b == 0x80000000u) b = 0u;  // -0.0 ranks with +0.0
-  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  const uint32_t b = __float_as_uint(f);
+  // positive: set the sign bit; negative: flip every bit
+  uint32_t key = b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
+  key += key == 0x7fffffffu ? 1u : 0u;  // -0.0 ranks with +0.0
+  return key;
 }
 
 constexpr int kStep = kWave * 4;  // elements one wave handles per step (one float4 per lane)
