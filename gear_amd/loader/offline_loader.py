@@ -91,6 +91,7 @@ class OfflineLoader(BasicLoader):
         sampler_cls = getattr(importlib.import_module("gear_amd.sampler"),
                               "%sSampler" % sampling_method)
         self._sampler = sampler_cls(self._mpu, seed=42)
+        self._sampler.indices_ascending = True   # arange + offset below
         self._indices = torch.arange(self._iset.local_capacity, dtype=torch.long,
                                      device=self._mpu.device) + self._iset.index_offset
         self.last_masks = None

@@ -30,6 +30,9 @@ class UniformSampler:
         self._mpu = mpu
         self._generator = torch.Generator(mpu.device)
         self._generator.manual_seed(seed)
+        # Set by a caller whose `indices` are ascending (a loader's arange + offset): positions
+        # that are already sorted then select sorted indices, and the final sort is skipped.
+        self.indices_ascending = False
 
     def sync_sample(self, indices, weights, batch_size, dirty_from=None):
         """dirty_from (an addition to the reference's signature, used by WeightedSampler): None =
@@ -41,9 +44,11 @@ class UniformSampler:
             return self._dp_rank_zero_sync(indices, weights, batch_size)
         return self._dp_rank_zero_sync(indices, weights, batch_size, dirty_from=dirty_from)
 
-    def _take_sorted(self, indices, positions):
+    def _take_sorted(self, indices, positions, positions_sorted=False):
         """sort(indices[positions]) on the device."""
         picked = ops.take_i64(indices, positions)
+        if positions_sorted and self.indices_ascending:
+            return picked
         bits = 63
         return ops.sort_i64(picked, key_bits=bits)
 
@@ -88,7 +93,7 @@ class WeightedSampler(UniformSampler):
         self._prefix = self._state.scan(weights, 0 if dirty_from is None else int(dirty_from))
         positions = ops.sample_sorted(self._prefix, draws, unit_uniforms=True)
         self.last_positions = positions
-        return self._take_sorted(indices, positions)
+        return self._take_sorted(indices, positions, positions_sorted=True)
 
     def sample_with_importance(self, indices, weights, batch_size, beta=0.4):
         """Draw a batch and its importance weights (N * P(i)) ** -beta / max over the batch.
@@ -112,4 +117,4 @@ class TopKSampler(UniformSampler):
 
     def select(self, indices, weights, draws, dirty_from=None):
         _, positions = ops.topk(weights, draws.numel(), sorted_by_value=False, want_values=False)
-        return self._take_sorted(indices, positions)
+        return self._take_sorted(indices, positions, positions_sorted=True)  # index-ordered
