@@ -59,7 +59,22 @@ TensorInfo tensor_info(const py::handle &t, const char *name, int64_t want_elem 
   return i;
 }
 
+// torch._C._cuda_getCurrentRawStream(device) where this torch has it (one C call), else
+// torch.cuda.current_stream().cuda_stream
 void *current_stream() {
+  // the two callables are kept for the life of the process (never destroyed: static py::objects
+  // would be released after the interpreter has gone)
+  static py::object *raw = nullptr, *getdev = nullptr;
+  static bool probed = false;
+  if (!probed) {
+    probed = true;
+    py::object c = torch_module().attr("_C");
+    if (py::hasattr(c, "_cuda_getCurrentRawStream") && py::hasattr(c, "_cuda_getDevice")) {
+      raw = new py::object(c.attr("_cuda_getCurrentRawStream"));
+      getdev = new py::object(c.attr("_cuda_getDevice"));
+    }
+  }
+  if (raw != nullptr) return reinterpret_cast<void *>((*raw)((*getdev)()).cast<uintptr_t>());
   py::object s = torch_module().attr("cuda").attr("current_stream")();
   return reinterpret_cast<void *>(s.attr("cuda_stream").cast<uintptr_t>());
 }

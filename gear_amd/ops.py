@@ -12,8 +12,22 @@ from . import _cabi
 from ._cabi import ColumnDesc, call, load
 
 
+# torch's C accessor for the raw current stream (a fraction of the cost of
+# torch.cuda.current_stream(), which builds a Stream object through several Python layers)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_cur_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
+def _stream_value(device=None):
+    if _raw_stream is not None and _cur_device is not None:
+        index = device.index if (device is not None and device.index is not None) \
+            else _cur_device()
+        return _raw_stream(index)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return ctypes.c_void_p(_stream_value())
 
 
 def _ptr(t):
@@ -53,7 +67,7 @@ class _Workspace:
         self._bufs = {}
 
     def get(self, tag, nbytes, device):
-        key = (tag, device, torch.cuda.current_stream(device).cuda_stream)
+        key = (tag, device, _stream_value(device))
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
