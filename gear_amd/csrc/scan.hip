@@ -3,7 +3,7 @@
 // Three kernels share the inner scan (each thread scans inside its 16-byte input vectors, row sums
 // go through a DPP wave scan, wave totals meet in LDS, results leave through LDS so that every store
 // instruction writes whole lines):
-//  * default, up to 2048 ranges (n <= 33.5 M fp32): two launches.  range_sum_kernel writes the sum
+//  * default, up to 8192 ranges (n <= 134 M fp32): two launches.  range_sum_kernel writes the sum
 //    of every range; scan_ranges_kernel<TWO = true> re-reads its range (now in L2 / MALL), adds
 //    the sums of all earlier ranges in a fixed order and writes the prefix.  No workgroup waits for
 //    another one.  On this multi-XCD part that is faster than the one-pass kernels: a ticket per
@@ -13,7 +13,7 @@
 //    numbers are handed out by an atomic ticket in launch order (every awaited predecessor is
 //    already running); a workgroup publishes the sum of its range in one agent-scope 64-bit store
 //    (kEmpty = not published, so no fence pairs) and sums ALL earlier ranges' words.
-//  * beyond 2048 ranges: scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone,
+//  * beyond that (and beyond 2048 ranges in the single-pass mode): scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone,
 //    incl[t] = sum of tiles 0..t; wave 0 looks back 64 predecessors at a time, ballots pick the
 //    nearest published inclusive value).
 #include "wave.hpp"
@@ -232,7 +232,8 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
 // it, and takes its exclusive prefix as the sum of ALL earlier ranges' aggregates (each thread
 // polls its share of them, fixed summation order).  Nobody waits for an inclusive value, so there
 // is no serial chain across the XCDs, and the result is bit-reproducible from run to run.
-constexpr int kMaxRanges = 2048;
+constexpr int kMaxRanges = 2048;     // single-pass variant: every thread polls 8 range sums
+constexpr int kMaxRangesTwo = 8192;  // two launches: every thread adds up to 32 range sums
 
 // Sum of every range, one workgroup per range: the first launch of the two-launch variant, in
 // which the scan launch below finds all aggregates ready (no ticket, no publishing, no polling).
@@ -334,7 +335,7 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
   }
   // sum of every earlier range (thread t takes ranges t, t+256, ...)
   // all of a thread's polls are issued together; only the ones not yet published are repeated
-  constexpr int kPolls = kMaxRanges / kBlock;
+  constexpr int kPolls = (TWO ? kMaxRangesTwo : kMaxRanges) / kBlock;
   uint64_t pv[kPolls];
 #pragma unroll
   for (int i = 0; i < kPolls; ++i) {
@@ -471,19 +472,19 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
       (reinterpret_cast<uintptr_t>(out) & 15))
     return GEAR_HIP_EALIGN;
   const int64_t row = (int64_t)kBlock * VE;
-  // Up to 2048 ranges of 2, 4, 8 or 16 rows of 256 vectors.  Default: two launches (range sums,
+  // Up to 8192 ranges of 2, 4, 8 or 16 rows of 256 vectors.  Default: two launches (range sums,
   // then the scan with every aggregate ready).  GEAR_HIP_SCAN_SINGLE_PASS=1 selects the one-pass
   // kernel with tickets and published aggregates instead (larger ranges, so that all workgroups
   // are resident together).
   const bool single_pass = env_int("GEAR_HIP_SCAN_SINGLE_PASS", 0) != 0;
-  const int64_t cap = single_pass ? 1024 : kMaxRanges;
+  const int64_t cap = single_pass ? 1024 : kMaxRanges;  // the largest ranges may be up to 8192
   if (!single_pass && ceil_div64(n, 2 * row) <= cap)
     return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, single_pass, first_changed);
   if (ceil_div64(n, 4 * row) <= cap)
     return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, single_pass, first_changed);
   if (ceil_div64(n, 8 * row) <= cap)
     return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, single_pass, first_changed);
-  if (ceil_div64(n, 16 * row) <= kMaxRanges)
+  if (ceil_div64(n, 16 * row) <= (single_pass ? kMaxRanges : kMaxRangesTwo))
     return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, single_pass, first_changed);
   const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);

@@ -12,7 +12,7 @@ torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
 
 SIZES = [1, 2, 3, 63, 64, 65, 255, 1023, 2047, 2048, 2049, 4095, 4096, 4097, 8191, 8192, 8193,
-         100_000, 1_000_000, 4_194_305, 10_000_003, 34_000_001]
+         100_000, 1_000_000, 4_194_305, 10_000_003, 34_000_001, 134_300_000]
 
 
 @pytest.fixture(params=["two_launch", "single_pass"])
