@@ -195,7 +195,7 @@ int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspa
  * with the same n, and since then only in[first_changed .. n) changed.  Then out[i] is
  * recomputed from the start of the range that holds first_changed onwards, reusing the range sums
  * kept in the workspace; the result is bit-identical to a full gear_hip_scan_f32_f64.
- * first_changed >= n: nothing to do; first_changed = 0, n > 33.5 M or
+ * first_changed >= n: nothing to do; first_changed = 0, n > 134 M or
  * GEAR_HIP_SCAN_SINGLE_PASS=1: a full scan. */
 int gear_hip_rescan_f32_f64(const float *in, double *out, int64_t n, int64_t first_changed,
                             void *workspace, size_t workspace_bytes, void *stream);
