@@ -301,3 +301,20 @@ def test_rescan_integer_valued_matches_oracle_exactly(oracle):
         announce("integer rescan first_changed=%d" % k)
         got = state.scan(dp, first_changed=k).cpu().numpy()
         assert np.array_equal(got, oracle.scan_f32_f64(p))
+
+
+def test_split_step_index():
+    """flat step index -> (trajectory, timestep, length = timestep + 1), optionally modulo the
+    number of steps in the table (BASELINE config 5 draws from 1e7 priorities over a 2e6-step
+    table)."""
+    from gear_amd import ops
+    rng = np.random.default_rng(4)
+    flat = rng.integers(0, 10_000_000, size=5000).astype(np.int64)
+    for T, modulo in ((1000, 0), (1000, 2_000_000), (7, 0), (1, 13)):
+        announce("split T=%d modulo=%d" % (T, modulo))
+        idxs, tss, lens = ops.split_step_index(_dev(flat), T, modulo)
+        torch.cuda.synchronize()
+        f = flat % modulo if modulo else flat
+        assert np.array_equal(idxs.cpu().numpy(), f // T)
+        assert np.array_equal(tss.cpu().numpy(), f % T)
+        assert np.array_equal(lens.cpu().numpy(), f % T + 1)
