@@ -522,13 +522,40 @@ def run_config3(args):
 
     ms_graph = _time_graph(torch, body, feed, args.steps, args.warmup)
     alg = 2 * B * span * sum(tab.step_bytes) + B * span
+    extra = _graph_extra(B, "windows/s", ms_graph)
+    if not args.no_cpu_baseline:
+        # CPU oracle on a bounded sample: the same sampler over all lengths, the gather on the
+        # first trajectories of the table (index taken modulo their number)
+        from oracle import oracle as orc
+        keep = min(2000, tab.capacity)
+        host = table[:keep * tab.traj_stride].cpu().numpy()
+        hl = lengths.cpu().numpy()
+        hd = [np.zeros((B, span * sb), np.uint8) for sb in tab.step_bytes]
+        crng = np.random.default_rng(3003)
+        t0 = time.perf_counter()
+        nrun = 0
+        while nrun < 3 or (time.perf_counter() - t0 < 3.0 and nrun < 2000):
+            pre = orc.scan_i64(hl)
+            traj = orc.sort_i64(orc.upper_bound_i64(pre, crng.random(B), unit_uniforms=True))
+            lens_h = hl[traj]
+            start = (crng.random(B) * (lens_h - (span - 1))).astype(np.int64)
+            for c in range(5):
+                orc.subcopy(host, traj % keep, start, lens_h, False, 0, span, tab.traj_stride,
+                            tab.step_bytes[c], tab.col_base(c), dst=hd[c], want_mask=(c == 0))
+            nrun += 1
+        cpu_ms = (time.perf_counter() - t0) * 1e3 / nrun
+        extra["cpu_baseline"] = {
+            "value": B / (cpu_ms * 1e-3), "unit": "windows/s", "cores": 1, "kind": "port",
+            "ms_per_step": cpu_ms,
+            "sample": "%d steps of int64 scan + 1024 searches + sort + 5-column gather with mask, "
+                      "table cut to its first %d trajectories" % (nrun, keep)}
     return _line(B / (ms * 1e-3), "windows/s", args, ms,
                  "config3: %d variable-length trajectories (T=1000), length-weighted int64 sampler, "
                  "1024 windows x 20 steps x 5 columns + uint8 mask" % tab.capacity,
                  {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": alg / (gms * 1e-3) / 1e9,
                   "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (gms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                   "avg_launch_ms": gms, "algorithmic_bytes": alg, "traffic": None},
-                 _graph_extra(B, "windows/s", ms_graph))
+                 extra)
 
 
 def run_config5(args):
@@ -613,6 +640,47 @@ def run_config5(args):
     torch.cuda.synchronize()
     link_gbps = payload / (a.elapsed_time(b) / 5 * 1e-3) / 1e9
     gather_gbps = payload / (parts["gather"] * 1e-3) / 1e9
+    extra5 = {}
+    if not args.no_cpu_baseline:
+        # CPU oracle, bounded: the maintenance step on the full 1e7 priorities, the gather on the
+        # first trajectories of the host table
+        from oracle import oracle as orc
+        keep = min(64, cap)
+        host = np.ctypeslib.as_array(
+            ctypes.cast(host_ptr, ctypes.POINTER(ctypes.c_uint8)), shape=(keep * tab.traj_stride,))
+        hp = pri.cpu().numpy().copy()
+        hidx = [t.cpu().numpy() for t in upd_idx]
+        hval = [t.cpu().numpy() for t in upd_val]
+        hd = [np.zeros((B, span * sb), np.uint8) for sb in tab.step_bytes]
+        crng = np.random.default_rng(3005)
+        parts_cpu = {n: 0.0 for n in names}
+        t_all = time.perf_counter()
+        nrun = 0
+        while nrun < 2 or (time.perf_counter() - t_all < 10.0 and nrun < 20):
+            t0 = time.perf_counter()
+            orc.scatter_f32(hp, hidx[nrun % 4], hval[nrun % 4])
+            t1 = time.perf_counter()
+            orc.topk_f32(hp, k, True)
+            t2 = time.perf_counter()
+            pre = orc.scan_f32_f64(hp)
+            t3 = time.perf_counter()
+            fl = orc.sort_i64(orc.upper_bound_f64(pre, crng.random(B, dtype=np.float32),
+                                                  unit_uniforms=True)) % (T * cap)
+            t4 = time.perf_counter()
+            for c in range(4):
+                orc.subcopy(host, (fl // T) % keep, fl % T, fl % T + 1, True, ofst, span,
+                            tab.traj_stride, tab.step_bytes[c], tab.col_base(c), dst=hd[c])
+            t5 = time.perf_counter()
+            for n_, d_ in zip(names, (t1 - t0, t2 - t1, t3 - t2, t4 - t3, t5 - t4)):
+                parts_cpu[n_] += d_ * 1e3
+            nrun += 1
+        cpu_ms = (time.perf_counter() - t_all) * 1e3 / nrun
+        extra5["cpu_baseline"] = {
+            "value": B / (cpu_ms * 1e-3), "unit": "windows/s", "cores": 1, "kind": "port",
+            "ms_per_step": cpu_ms, "parts_ms": {n_: v / nrun for n_, v in parts_cpu.items()},
+            "sample": "%d steps: scatter 65536, top-65536 of 1e7, fp64 rescan of 1e7, 2048 draws, "
+                      "4-column gather from the first %d trajectories of the host table"
+                      % (nrun, keep)}
     lib.gear_hip_host_free(host_ptr)
     return _line(B / (ms * 1e-3), "windows/s", args, ms,
                  "config5: %d-step Atari-shape table in pinned host memory (%.1f GB, zero-copy), per "
@@ -624,9 +692,9 @@ def run_config5(args):
                   "algorithmic_bytes": payload,
                   "peak_source": "pinned hipMemcpyAsync H2D of the same bytes in this run",
                   "traffic": None},
-                 {"parts_ms": parts,
-                  "maintenance": {"topk_GBps_one_read": 4 * npri / (parts["topk"] * 1e-3) / 1e9,
-                                  "rescan_GBps": 12 * npri / (parts["scan"] * 1e-3) / 1e9}})
+                 dict(extra5, parts_ms=parts,
+                      maintenance={"topk_GBps_one_read": 4 * npri / (parts["topk"] * 1e-3) / 1e9,
+                                   "rescan_GBps": 12 * npri / (parts["scan"] * 1e-3) / 1e9}))
 
 
 def main():
