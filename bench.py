@@ -121,7 +121,9 @@ def run_config4(args):
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    gather_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    launch_ms = sorted(a.elapsed_time(b) for a, b in ev)
+    gather_ms = sum(launch_ms) / args.steps
+    pct = lambda q: launch_ms[min(len(launch_ms) - 1, int(q * len(launch_ms)))]
 
     # The same K steps again with the sampler of batch i+1 enqueued on a second stream while
     # batch i is being gathered (what a prefetching loader does); reported next to the serial
@@ -210,7 +212,8 @@ def run_config4(args):
         "step_frac_of_hbm_peak": alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "kernel": "subcopy_multi_kernel", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "avg_launch_ms": gather_ms, "algorithmic_bytes": alg_bytes,
+                     "avg_launch_ms": gather_ms, "launch_ms_p10_p50_p90": [pct(0.1), pct(0.5), pct(0.9)],
+                     "algorithmic_bytes": alg_bytes,
                      "traffic": args.traffic_bytes if args.traffic_bytes is not None else
                      (MEASURED_GATHER_TRAFFIC_BYTES if cap == 1000 else None)},
     }
