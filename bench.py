@@ -185,8 +185,16 @@ def run_config4(args):
 
         ms_lib = timed_ms(lambda: ops.copy(table, ydst, zero, zero, payload))
         ms_torch = timed_ms(lambda: ydst.copy_(ysrc))
+        # one-directional streams through torch's own kernels: a fill (write only) and a sum
+        # (read only) over the same number of bytes
+        n8 = payload // 8
+        y64 = ydst[:n8 * 8].view(torch.int64)
+        ms_fill = timed_ms(lambda: y64.fill_(1))
+        ms_sum = timed_ms(lambda: y64.sum())
         yard = {"contiguous_copy_slice_kernel_GBps": alg_bytes / (ms_lib * 1e-3) / 1e9,
                 "contiguous_copy_torch_GBps": alg_bytes / (ms_torch * 1e-3) / 1e9,
+                "write_only_torch_fill_GBps": n8 * 8 / (ms_fill * 1e-3) / 1e9,
+                "read_only_torch_sum_GBps": n8 * 8 / (ms_sum * 1e-3) / 1e9,
                 "gather_vs_contiguous_copy": ms_lib / gather_ms,
                 "what": "%d bytes read + written as one contiguous piece, same run" % payload}
         del ydst
