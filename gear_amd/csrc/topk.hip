@@ -18,9 +18,14 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kMaxRanges = 2048;  // workgroups of the compaction launches
-constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kCompactThreads = 512;  // threads of a compaction workgroup (256: +2.5 us at n = 1e7)
+constexpr int kWavesPerBlock = kCompactThreads / kWave;
 constexpr int kHistBins = 2048;
-constexpr int kMaxHistBlocks = 512;
+// Histogram launches: one 1024-thread workgroup per CU.  Fewer, fatter workgroups mean fewer
+// flush atomics per bin and fewer workgroups that pick the previous bin (measured at n = 1e7:
+// 512 x 256 threads 60.8 us for the whole top-k, 256 x 512 56.0, 512 x 1024 54.9, 256 x 1024 53.1).
+constexpr int kMaxHistBlocks = 256;
+constexpr int kHistThreads = 1024;
 
 struct State {
   uint32_t prefix[3];  // key bits decided after pass 0, 1, 2 (right-aligned)
@@ -104,11 +109,11 @@ __global__ void zero_kernel(uint32_t *p, int64_t words) {
 struct Pick {
   uint32_t prefix, k_rem;
 };
-template <int PASS>
+template <int PASS, int THREADS = kBlock>
 __device__ __forceinline__ Pick pick_bin(int64_t k, State *state, const uint32_t *hist) {
   constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
-  constexpr int kPerThread = kBinsHere / kBlock;
-  __shared__ uint32_t wsum[kBlock / kWave];
+  constexpr int kPerThread = kBinsHere / THREADS;
+  __shared__ uint32_t wsum[THREADS / kWave];
   __shared__ Pick s_pick;
   const int tid = threadIdx.x;
   const uint32_t prefix = PASS == 0 ? 0u : state->prefix[PASS == 0 ? 0 : PASS - 1];
@@ -149,17 +154,17 @@ __device__ __forceinline__ Pick pick_bin(int64_t k, State *state, const uint32_t
 // add their non-empty bins to the global histogram of this pass (hist; the previous pass's is
 // at hist - kHistBins); the bin of the previous pass is picked by every workgroup for itself.
 template <int PASS>
-__global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__restrict__ p,
+__global__ __launch_bounds__(kHistThreads) void select_hist_kernel(const float *__restrict__ p,
                                                              int64_t n, int64_t k, State *state,
                                                              uint32_t *hist) {
   constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
   typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
   __shared__ uint32_t h[kBinsHere];
   const int tid = threadIdx.x;
-  for (int i = tid; i < kBinsHere; i += kBlock) h[i] = 0;
+  for (int i = tid; i < kBinsHere; i += kHistThreads) h[i] = 0;
   uint32_t prefix = 0u;
-  if (PASS == 1) prefix = pick_bin<0>(k, state, hist - kHistBins).prefix;
-  if (PASS == 2) prefix = pick_bin<1>(k, state, hist - kHistBins).prefix;
+  if (PASS == 1) prefix = pick_bin<0, kHistThreads>(k, state, hist - kHistBins).prefix;
+  if (PASS == 2) prefix = pick_bin<1, kHistThreads>(k, state, hist - kHistBins).prefix;
   __syncthreads();
 
   // Passes 1 and 2 count only the keys that start with `prefix`: about 1 % of the input.  Whether
@@ -181,18 +186,18 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__rest
   };
   const int64_t nvec = n >> 2;
   constexpr int kLoads = 4;  // 16-byte loads in flight per thread
-  for (int64_t v0 = (int64_t)blockIdx.x * kBlock * kLoads + tid; v0 < nvec;
-       v0 += (int64_t)gridDim.x * kBlock * kLoads) {
+  for (int64_t v0 = (int64_t)blockIdx.x * kHistThreads * kLoads + tid; v0 < nvec;
+       v0 += (int64_t)gridDim.x * kHistThreads * kLoads) {
     f4 q[kLoads];
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) {
-      const int64_t v = v0 + (int64_t)u * kBlock;
+      const int64_t v = v0 + (int64_t)u * kHistThreads;
       q[u] = f4{0.0f, 0.0f, 0.0f, 0.0f};
       if (v < nvec) q[u] = *reinterpret_cast<const f4 *>(p + (v << 2));
     }
 #pragma unroll
     for (int u = 0; u < kLoads; ++u) {
-      if (v0 + (int64_t)u * kBlock < nvec) {
+      if (v0 + (int64_t)u * kHistThreads < nvec) {
         count(q[u][0]);
         count(q[u][1]);
         count(q[u][2]);
@@ -202,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const float *__rest
   }
   if (blockIdx.x == 0 && tid < (int)(n & 3)) count(p[(nvec << 2) + tid]);
   __syncthreads();
-  for (int i = tid; i < kBinsHere; i += kBlock)
+  for (int i = tid; i < kBinsHere; i += kHistThreads)
     if (h[i]) atomicAdd(&hist[i], h[i]);
 }
 
@@ -224,7 +229,7 @@ __device__ __forceinline__ void load_quad(const float *__restrict__ p, int64_t e
   }
 }
 
-__global__ __launch_bounds__(kBlock) void count_ranges_kernel(
+__global__ __launch_bounds__(kCompactThreads) void count_ranges_kernel(
     const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist2,
     int64_t wave_len, uint64_t *__restrict__ wave_counts, uint64_t *__restrict__ block_counts,
     uint32_t *__restrict__ lists, int list_cap) {
@@ -241,7 +246,7 @@ __global__ __launch_bounds__(kBlock) void count_ranges_kernel(
   float q[kAhead][4];
 #pragma unroll
   for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
-  const float thr_f = key_to_float(pick_bin<2>(k, state, hist2).prefix);
+  const float thr_f = key_to_float(pick_bin<2, kCompactThreads>(k, state, hist2).prefix);
   uint32_t gt = 0, eq = 0;
   for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
     // the next batch of loads is in flight while this one is classified and listed
@@ -310,7 +315,7 @@ __global__ __launch_bounds__(kBlock) void count_ranges_kernel(
 }
 
 template <bool DIRECT>
-__global__ __launch_bounds__(kBlock) void write_ranges_kernel(
+__global__ __launch_bounds__(kCompactThreads) void write_ranges_kernel(
     const float *__restrict__ p, int64_t n, const State *state, int64_t wave_len,
     const uint64_t *__restrict__ wave_counts, const uint64_t *__restrict__ block_counts,
     const uint32_t *__restrict__ lists, int list_cap, uint32_t *__restrict__ ckey,
@@ -331,7 +336,7 @@ __global__ __launch_bounds__(kBlock) void write_ranges_kernel(
   const uint32_t need_eq = state->k_rem[2];
 
   int64_t part = 0;
-  for (int j = tid; j < (int)blockIdx.x; j += kBlock) part += (int64_t)block_counts[j];
+  for (int j = tid; j < (int)blockIdx.x; j += kCompactThreads) part += (int64_t)block_counts[j];
   const int64_t pw = wave_sum(part);
   if (lane == 0) red[wave] = pw;
   __syncthreads();
@@ -450,13 +455,13 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   const int64_t zero_words = (int64_t)(l.desc / 4);  // header + histograms
   zero_kernel<<<dim3((unsigned)ceil_div64(zero_words, 256)), dim3(256), 0, st>>>(
       reinterpret_cast<uint32_t *>(ws), zero_words);
-  int64_t hblocks = ceil_div64(n, (int64_t)kBlock * 4 * 4);
+  int64_t hblocks = ceil_div64(n, (int64_t)kHistThreads * 4 * 4);
   if (hblocks < 1) hblocks = 1;
   if (hblocks > kMaxHistBlocks) hblocks = kMaxHistBlocks;
-  const dim3 hgrid((unsigned)hblocks), block(kBlock);
-  select_hist_kernel<0><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist);
-  select_hist_kernel<1><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist + kHistBins);
-  select_hist_kernel<2><<<hgrid, block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins);
+  const dim3 hgrid((unsigned)hblocks), hblock(kHistThreads), block(kBlock);
+  select_hist_kernel<0><<<hgrid, hblock, 0, st>>>(priorities, n, k, state, hist);
+  select_hist_kernel<1><<<hgrid, hblock, 0, st>>>(priorities, n, k, state, hist + kHistBins);
+  select_hist_kernel<2><<<hgrid, hblock, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
 
   uint32_t *ckey = reinterpret_cast<uint32_t *>(ws + l.ckey);
@@ -467,16 +472,16 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   uint32_t *lists = reinterpret_cast<uint32_t *>(ws + l.lists);
   uint64_t *wave_counts = reinterpret_cast<uint64_t *>(ws + l.desc);
   uint64_t *block_counts = wave_counts + (size_t)kMaxRanges * kWavesPerBlock;
-  const dim3 cgrid((unsigned)ranges);
-  count_ranges_kernel<<<cgrid, block, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins,
+  const dim3 cgrid((unsigned)ranges), cblock(kCompactThreads);
+  count_ranges_kernel<<<cgrid, cblock, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins,
                                                wave_len, wave_counts, block_counts, lists,
                                                (int)g.list_cap);
   if (direct)
-    write_ranges_kernel<true><<<cgrid, block, 0, st>>>(priorities, n, state, wave_len, wave_counts,
+    write_ranges_kernel<true><<<cgrid, cblock, 0, st>>>(priorities, n, state, wave_len, wave_counts,
                                                        block_counts, lists, (int)g.list_cap, ckey,
                                                        cidx, values_out, indices_out);
   else
-    write_ranges_kernel<false><<<cgrid, block, 0, st>>>(priorities, n, state, wave_len,
+    write_ranges_kernel<false><<<cgrid, cblock, 0, st>>>(priorities, n, state, wave_len,
                                                         wave_counts, block_counts, lists,
                                                         (int)g.list_cap, ckey, cidx, values_out,
                                                         indices_out);
