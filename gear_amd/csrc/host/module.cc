@@ -428,7 +428,7 @@ PYBIND11_MODULE(_libgear, libgear) {
             return table;
           }));
 
-  auto span64 = [](const py::object &o, const char *name) {
+  auto span64 = [](const py::object &o, const char * /*name*/) {
     if (py::isinstance<Int64Span>(o)) return o.cast<Int64Span>();
     return span_from_tensor<DataType::kInt64>(o);
   };

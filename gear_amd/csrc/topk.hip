@@ -449,7 +449,6 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   char *ws = static_cast<char *>(workspace);
   State *state = reinterpret_cast<State *>(ws);
   uint32_t *hist = reinterpret_cast<uint32_t *>(ws + l.hist);
-  uint64_t *desc = reinterpret_cast<uint64_t *>(ws + l.desc);
   hipStream_t st = as_stream(stream);
 
   const int64_t zero_words = (int64_t)(l.desc / 4);  // header + histograms
