@@ -109,11 +109,21 @@ __global__ __launch_bounds__(kBlock) void digit_scan_kernel(uint32_t *__restrict
 
 // FUSED: `table` holds this digit's raw tile-major counts.  Otherwise `table` holds the
 // digit-major row prefixes and `totals` the digit totals.
-template <typename K, typename V, bool HAS_V, bool FUSED>
+// What the LAST digit's scatter does with a sorted pair instead of storing it to kout/vout: a
+// caller may pass its own functor (kActive = true, operator()(position, key, value)) to fuse the
+// kernel that would otherwise read the sorted arrays once more.
+struct StoreSorted {
+  static constexpr bool kActive = false;
+  template <typename K, typename V>
+  __device__ __forceinline__ void operator()(uint32_t, K, V) const {}
+};
+
+template <typename K, typename V, bool HAS_V, bool FUSED, typename Final>
 __global__ __launch_bounds__(kBlock) void scatter_kernel(
     const K *__restrict__ kin, const V *__restrict__ vin, K *__restrict__ kout,
     V *__restrict__ vout, int64_t num, int shift, uint32_t dmask, int rounds, int64_t ntiles,
-    const uint32_t *__restrict__ table, const uint32_t *__restrict__ totals) {
+    const uint32_t *__restrict__ table, const uint32_t *__restrict__ totals, Final fin,
+    int last) {
   constexpr int kSub = 4;                  // rounds ranked together: independent ballot chains
   constexpr int kSlots = kSub * kWaves;    // (round, wave) slots of the count table
   __shared__ uint32_t base[kBins];
@@ -234,8 +244,12 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(
     for (int q = 0; q < kSub; ++q) {
       if (valid[q]) {
         const uint32_t pos = wpre[q * kWaves + wave][d[q]] + (uint32_t)rank[q];
-        kout[pos] = kcur[q];
-        if (HAS_V) vout[pos] = vcur[q];
+        if (Final::kActive && last) {
+          fin(pos, kcur[q], vcur[q]);
+        } else {
+          kout[pos] = kcur[q];
+          if (HAS_V) vout[pos] = vcur[q];
+        }
       }
     }
     // the next use of wpre is ordered behind this scatter by the barrier after the next ballots
@@ -355,9 +369,11 @@ __global__ void copy_kernel(const T *__restrict__ in, T *__restrict__ out, int64
 // Sorts bits [begin_bit, end_bit) of the keys ascending, stable.  kin/vin are not modified; the
 // result lands in kout/vout; ktmp/vtmp are scratch of the same size; hist has hist_bytes(num).
 // vin == nullptr sorts keys only.  num < 2^32.
-template <typename K, typename V>
+// `fin` (see StoreSorted) replaces the stores of the last digit on the radix path; batches of at
+// most kRankMax keys take the ranking sort, which ignores it (the caller checks num).
+template <typename K, typename V, typename Final = StoreSorted>
 int sort_pairs(const K *kin, K *kout, const V *vin, V *vout, K *ktmp, V *vtmp, int64_t num,
-               int begin_bit, int end_bit, uint32_t *hist, hipStream_t st) {
+               int begin_bit, int end_bit, uint32_t *hist, hipStream_t st, Final fin = Final()) {
   if (num <= 0) return 0;
   if (num >= (1ll << 32)) return GEAR_HIP_ERANGE;
   const Plan p = plan(num);
@@ -395,25 +411,30 @@ int sort_pairs(const K *kin, K *kout, const V *vin, V *vout, K *ktmp, V *vtmp, i
     const uint32_t dmask = end_bit - shift >= 8 ? 255u : ((1u << (end_bit - shift)) - 1u);
     K *kdst = to_out ? kout : ktmp;
     V *vdst = to_out ? vout : vtmp;
+    const int last = pass + 1 == passes ? 1 : 0;
     if (p.fused) {
       hist_kernel<K, true><<<grid, block, 0, st>>>(ksrc, num, shift, dmask, p.rounds, p.ntiles,
                                                    table);
       if (has_v)
-        scatter_kernel<K, V, true, true><<<grid, block, 0, st>>>(
-            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, nullptr);
+        scatter_kernel<K, V, true, true, Final><<<grid, block, 0, st>>>(
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, nullptr, fin,
+            last);
       else
-        scatter_kernel<K, V, false, true><<<grid, block, 0, st>>>(
-            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, nullptr);
+        scatter_kernel<K, V, false, true, Final><<<grid, block, 0, st>>>(
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, nullptr, fin,
+            last);
     } else {
       hist_kernel<K, false><<<grid, block, 0, st>>>(ksrc, num, shift, dmask, p.rounds, p.ntiles,
                                                     table);
       digit_scan_kernel<<<dim3(kBins), block, 0, st>>>(table, p.ntiles, totals);
       if (has_v)
-        scatter_kernel<K, V, true, false><<<grid, block, 0, st>>>(
-            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, totals);
+        scatter_kernel<K, V, true, false, Final><<<grid, block, 0, st>>>(
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, totals, fin,
+            last);
       else
-        scatter_kernel<K, V, false, false><<<grid, block, 0, st>>>(
-            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, totals);
+        scatter_kernel<K, V, false, false, Final><<<grid, block, 0, st>>>(
+            ksrc, vsrc, kdst, vdst, num, shift, dmask, p.rounds, p.ntiles, table, totals, fin,
+            last);
     }
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     ksrc = kdst;

@@ -417,6 +417,18 @@ __global__ __launch_bounds__(kCompactThreads) void write_ranges_kernel(
   }
 }
 
+// Final store of the value-ordered form, fused into the last digit of the candidate sort.
+struct EmitSorted {
+  static constexpr bool kActive = true;
+  const float *p;
+  float *values;
+  int64_t *indices;
+  __device__ __forceinline__ void operator()(uint32_t pos, uint32_t, uint32_t index) const {
+    indices[pos] = (int64_t)index;
+    if (values) values[pos] = p[index];
+  }
+};
+
 __global__ __launch_bounds__(kBlock) void emit_kernel(const float *__restrict__ p,
                                                       const uint32_t *__restrict__ sidx, int64_t k,
                                                       float *__restrict__ values_out,
@@ -488,10 +500,17 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   if (direct) return 0;
   uint32_t *skey = reinterpret_cast<uint32_t *>(ws + l.skey);
   uint32_t *sidx = reinterpret_cast<uint32_t *>(ws + l.sidx);
-  int rc = radix::sort_pairs<uint32_t, uint32_t>(
-      ckey, skey, cidx, sidx, reinterpret_cast<uint32_t *>(ws + l.tkey),
-      reinterpret_cast<uint32_t *>(ws + l.tidx), k, 0, 32,
-      reinterpret_cast<uint32_t *>(ws + l.shist), st);
+  uint32_t *tkey = reinterpret_cast<uint32_t *>(ws + l.tkey);
+  uint32_t *tidx = reinterpret_cast<uint32_t *>(ws + l.tidx);
+  uint32_t *shist = reinterpret_cast<uint32_t *>(ws + l.shist);
+  if (k > radix::kRankMax) {
+    // radix path: the last digit's scatter writes values_out / indices_out itself
+    const EmitSorted fin{priorities, values_out, indices_out};
+    return radix::sort_pairs<uint32_t, uint32_t, EmitSorted>(ckey, skey, cidx, sidx, tkey, tidx, k,
+                                                             0, 32, shist, st, fin);
+  }
+  int rc = radix::sort_pairs<uint32_t, uint32_t>(ckey, skey, cidx, sidx, tkey, tidx, k, 0, 32,
+                                                 shist, st);
   if (rc) return rc;
   emit_kernel<<<dim3((unsigned)ceil_div64(k, kBlock)), block, 0, st>>>(priorities, sidx, k,
                                                                       values_out, indices_out);
