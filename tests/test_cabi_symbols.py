@@ -66,3 +66,18 @@ def test_missing_library_is_loud(tmp_path, monkeypatch):
     monkeypatch.setattr(_cabi, "LIB_PATH", str(tmp_path / "libgearhip.so"))
     with pytest.raises(ImportError):
         _cabi.load()
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/gear_hip.h is the boundary a C, Go (cgo) or Rust binding would consume: it must
+    compile as C99 on its own."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "gear_hip.h"\nint main(void) { return GEAR_HIP_ABI_VERSION < 0; }\n')
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, "-c",
+                    str(src), "-o", str(tmp_path / "use_header.o")], check=True)
