@@ -73,6 +73,8 @@ def test_header_is_plain_c(tmp_path):
     compile as C99 on its own."""
     import shutil
     import subprocess
+
+    import pytest
     gcc = shutil.which("gcc")
     if gcc is None:
         pytest.skip("no gcc")
