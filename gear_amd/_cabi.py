@@ -56,6 +56,8 @@ SIGNATURES = {
     "gear_hip_take_i64": (c_int, [c_void_p, c_i64, c_void_p, c_i64, c_i64, c_void_p, c_void_p]),
     "gear_hip_scan_workspace_bytes": (c_size_t, [c_i64]),
     "gear_hip_scan_f32_f64": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_size_t, c_void_p]),
+    "gear_hip_scan_static_max_n": (c_i64, []),
+    "gear_hip_scan_f32_f64_static": (c_int, [c_void_p, c_void_p, c_i64, c_void_p]),
     "gear_hip_rescan_f32_f64": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_void_p, c_size_t,
                                         c_void_p]),
     "gear_hip_scan_f32_f32": (c_int, [c_void_p, c_void_p, c_i64, c_void_p, c_size_t, c_void_p]),

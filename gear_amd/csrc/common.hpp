@@ -38,6 +38,11 @@ int env_int(const char *name, int dflt);
 
 __host__ __device__ inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Looks up, for the current device, the address of the static device array behind
+// gear_hip_scan_f32_f64_static (scan.hip); called by gear_hip_set_device so that the lookup
+// happens at set-up rather than inside the first hot-path call.
+int scan_static_init();
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace gearhip

@@ -25,7 +25,7 @@ extern "C" int gear_hip_set_device(int device_id) {
   int current = -1;
   GEARHIP_CHECK(hipGetDevice(&current));
   if (current != device_id) GEARHIP_CHECK(hipSetDevice(device_id));
-  return 0;
+  return scan_static_init();
 }
 
 extern "C" int gear_hip_device_count(int *count) {

@@ -16,6 +16,8 @@
 //  * beyond that (and beyond 2048 ranges in the single-pass mode): scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone,
 //    incl[t] = sum of tiles 0..t; wave 0 looks back 64 predecessors at a time, ballots pick the
 //    nearest published inclusive value).
+#include <atomic>
+
 #include "wave.hpp"
 
 namespace gearhip {
@@ -511,6 +513,61 @@ extern "C" int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, vo
                                      size_t workspace_bytes, void *stream) {
   return launch_scan<float, double, double, 4>(in, out, n, workspace, workspace_bytes,
                                                as_stream(stream));
+}
+
+// ---- the scan with its workspace in a static device array ---------------------------------------
+// For callers that cannot allocate device memory (a stream under graph capture, a serving loop
+// with a frozen memory pool): the range sums live in a file-scope device array instead of a
+// caller-supplied workspace.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the device address it yields (one per GPU, each GPU holds its own copy)
+// is what the kernels and every host-side use receive.
+namespace gearhip {
+namespace {
+
+constexpr int64_t kStaticMaxN = 1ll << 27;  // 134 217 728 priorities
+constexpr size_t kStaticBytes = kHeaderBytes + (size_t)(kStaticMaxN / (kRows * kBlock * 2)) * 16;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void **ptr) {
+  int dev = -1;
+  GEARHIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return GEAR_HIP_ERANGE;
+  void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    GEARHIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (p == nullptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // every thread finds the same address
+  }
+  *ptr = p;
+  return 0;
+}
+
+}  // namespace
+
+int scan_static_init() {
+  void *p = nullptr;
+  return static_scratch(&p);
+}
+
+}  // namespace gearhip
+
+extern "C" int64_t gear_hip_scan_static_max_n(void) { return kStaticMaxN; }
+
+extern "C" int gear_hip_scan_f32_f64_static(const float *in, double *out, int64_t n,
+                                            void *stream) {
+  if (n < 0) return GEAR_HIP_EINVAL;
+  if (n > kStaticMaxN) return GEAR_HIP_ERANGE;
+  if (n == 0) return 0;
+  void *ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc) return rc;
+  static_assert(kStaticBytes >= kHeaderBytes + 16, "scratch holds at least one range");
+  if (kStaticBytes < scan_ws_bytes(n)) return GEAR_HIP_ERANGE;
+  return launch_scan<float, double, double, 4>(in, out, n, ws, kStaticBytes, as_stream(stream));
 }
 
 extern "C" int gear_hip_rescan_f32_f64(const float *in, double *out, int64_t n,

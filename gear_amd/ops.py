@@ -219,6 +219,19 @@ def prefix_sum(priorities, out=None):
     return out
 
 
+def prefix_sum_static(priorities, out):
+    """fp32[n] -> fp64 prefix[n] into the caller's `out` with no allocation anywhere: the range
+    sums live in the library's static device array (gear_hip_scan_f32_f64_static).  Calls that
+    overlap on one GPU share that array and race."""
+    _need(priorities, torch.float32, "priorities")
+    _need(out, torch.float64, "out")
+    n = priorities.numel()
+    if out.numel() < n:
+        raise ValueError("out is too small")
+    call("gear_hip_scan_f32_f64_static", _ptr(priorities), _ptr(out), n, _stream())
+    return out
+
+
 class PrefixState:
     """The fp64 prefix of ONE priority array together with a workspace of its own, so that the
     range sums of the last scan survive other scans and a rescan can start at the first changed

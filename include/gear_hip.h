@@ -188,6 +188,18 @@ size_t gear_hip_scan_workspace_bytes(int64_t n);
 int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspace,
                           size_t workspace_bytes, void *stream);
 
+/* gear_hip_scan_f32_f64 for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses with a frozen memory pool.  It has no counterpart in
+ * the reference.  The range sums that the other entry point keeps in the caller's workspace live
+ * in a static device array inside the library (about 1 MiB per GPU, held until the process ends);
+ * the call allocates and frees nothing.  Same result, bit for bit, as gear_hip_scan_f32_f64.
+ * n <= gear_hip_scan_static_max_n() (2^27 = 134 217 728), else GEAR_HIP_ERANGE.
+ * The array's address is looked up once per device, by gear_hip_set_device or by the first call
+ * on that device.  All calls on one GPU share the array: calls that overlap on one GPU (two
+ * streams, two threads) race; serialise them or use the workspace form. */
+int64_t gear_hip_scan_static_max_n(void);
+int gear_hip_scan_f32_f64_static(const float *in, double *out, int64_t n, void *stream);
+
 /* Incremental form for the online priority path (priorities of a few trajectories change between
  * batches: SharedMemoryIndexServer::update, src/index/server.cc:175-180, and
  * WeightUpdateRequestArray, src/index/request.cc:41-75; the reference has no prefix to maintain).

@@ -54,6 +54,11 @@ def test_error_paths_without_gpu():
     assert lib.gear_hip_subcopy(None, None, 0, None, None, None, 0, 0, 1, 1, 1, 0, 1, 1, None,
                                 None) == 0
     assert lib.gear_hip_scan_f32_f64(None, None, 0, None, 0, None) == 0
+    # the allocation-free scan checks its size limit before it touches the device
+    assert lib.gear_hip_scan_static_max_n() == 1 << 27
+    assert lib.gear_hip_scan_f32_f64_static(None, None, (1 << 27) + 1, None) == -3
+    assert lib.gear_hip_scan_f32_f64_static(None, None, -1, None) == -1
+    assert lib.gear_hip_scan_f32_f64_static(None, None, 0, None) == 0
     # workspace queries are pure host arithmetic
     assert lib.gear_hip_scan_workspace_bytes(1_000_000) >= 256 + 16 * 245
     assert lib.gear_hip_topk_workspace_bytes(10_000_000, 65_536) > 6 * 4 * 65_536
