@@ -43,7 +43,9 @@ def install_as_gear():
         sys.modules.setdefault("gear." + sub, mod)
         setattr(me, sub, mod)
     # modules that pickled objects of the reference name (SharedDatasetMeta, IndexMeta)
-    for sub in ("dataset.shared_dataset", "sampler.global_sampler", "loader.offline_loader",
-                "loader.basic_loader"):
+    for sub in ("dataset.shared_dataset", "sampler.global_sampler", "loader.offline_loader"):
         sys.modules.setdefault("gear." + sub, importlib.import_module(__name__ + "." + sub))
+    # BasicLoader lives beside OfflineLoader here
+    sys.modules.setdefault("gear.loader.basic_loader",
+                           importlib.import_module(__name__ + ".loader.offline_loader"))
     return me

@@ -468,14 +468,26 @@ PYBIND11_MODULE(_libgear, libgear) {
                if (mi.numel < a.numel * w.span) throw std::runtime_error("mask is smaller than [num, length]");
                mp = static_cast<uint8_t *>(mi.ptr);
              }
+             // one-column form of the checked launch: the handler knows the table's extent, so
+             // an index outside it gathers nothing instead of reading outside the table
+             gear_hip_column_desc desc;
+             desc.dst = d.ptr;
+             desc.mask_out = mp;
+             desc.ofst = w.ofst;
+             desc.span = w.span;
+             desc.step_bytes = w.step_bytes;
+             desc.col_base = w.col_base;
+             desc.dst_stride = w.dst_stride;
+             desc.pad_head = w.pad_head ? 1 : 0;
+             desc.zero_fill = zero_fill ? 1 : 0;
              check_hip("subcopy",
-                       gear_hip_subcopy(h.impl.device_base(), d.ptr, a.numel,
-                                        static_cast<const int64_t *>(a.ptr),
-                                        static_cast<const int64_t *>(b.ptr),
-                                        static_cast<const int64_t *>(c.ptr), w.pad_head ? 1 : 0, w.ofst,
-                                        w.span, (int64_t)h.impl.table().trajectory_stride(),
-                                        w.step_bytes, w.col_base, w.dst_stride, zero_fill ? 1 : 0, mp,
-                                        current_stream()));
+                       gear_hip_subcopy_multi_checked(
+                           h.impl.device_base(), a.numel, static_cast<const int64_t *>(a.ptr),
+                           static_cast<const int64_t *>(b.ptr), static_cast<const int64_t *>(c.ptr),
+                           (int64_t)h.impl.table().trajectory_stride(),
+                           (int64_t)h.impl.table().table_spec().capacity,
+                           (int64_t)h.impl.table().table_spec().trajectory_length, &desc, 1,
+                           current_stream()));
            },
            py::arg("indices"), py::arg("timesteps"), py::arg("lengths"), py::arg("column"),
            py::arg("dst"), py::arg("zero_fill") = false, py::arg("mask") = py::none())

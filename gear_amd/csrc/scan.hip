@@ -17,6 +17,7 @@
 //    incl[t] = sum of tiles 0..t; wave 0 looks back 64 predecessors at a time, ballots pick the
 //    nearest published inclusive value).
 #include <atomic>
+#include <type_traits>
 
 #include "wave.hpp"
 
@@ -25,7 +26,7 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kRows = 4;
-constexpr uint64_t kEmpty = ~0ull;  // not a sum of fp32-derived doubles, not a non-negative int64
+constexpr uint64_t kEmpty = ~0ull;  // no fp64 sum of fp32 values has this bit pattern (fp64 scans only)
 constexpr size_t kHeaderBytes = 256;
 
 template <typename Acc> struct Bits;
@@ -478,7 +479,11 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
   // then the scan with every aggregate ready).  GEAR_HIP_SCAN_SINGLE_PASS=1 selects the one-pass
   // kernel with tickets and published aggregates instead (larger ranges, so that all workgroups
   // are resident together).
-  const bool single_pass = env_int("GEAR_HIP_SCAN_SINGLE_PASS", 0) != 0;
+  // The kernels in which a workgroup waits for another one mark "not published yet" with the
+  // word kEmpty, which no fp64 sum of fp32 values can equal but an int64 sum can (-1): int64
+  // scans therefore always take the two launches, in which nobody waits, and stop at their limit.
+  constexpr bool kMayWait = std::is_same<Acc, double>::value;
+  const bool single_pass = kMayWait && env_int("GEAR_HIP_SCAN_SINGLE_PASS", 0) != 0;
   const int64_t cap = single_pass ? 1024 : kMaxRanges;  // the largest ranges may be up to 8192
   if (!single_pass && ceil_div64(n, 2 * row) <= cap)
     return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, single_pass, first_changed);
@@ -488,6 +493,7 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
     return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, single_pass, first_changed);
   if (ceil_div64(n, 16 * row) <= (single_pass ? kMaxRanges : kMaxRangesTwo))
     return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, single_pass, first_changed);
+  if (!kMayWait) return GEAR_HIP_ERANGE;
   const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
   uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);

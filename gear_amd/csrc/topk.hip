@@ -128,6 +128,12 @@ __device__ __forceinline__ Pick pick_bin(int64_t k, State *state, const uint32_t
   }
   const int inc = wave_inclusive_sum(tsum);
   if ((tid & 63) == 63) wsum[tid >> 6] = (uint32_t)inc;
+  // fallback when no bin holds the k_rem-th key (only possible with NaN priorities, which the
+  // float compares of the later passes do not count): the lowest bin, nothing taken off k_rem
+  if (tid == 0) {
+    s_pick.prefix = PASS == 0 ? 0u : (PASS == 1 ? (prefix << 11) : (prefix << 10));
+    s_pick.k_rem = k_rem;
+  }
   __syncthreads();
   uint32_t running = (uint32_t)(inc - tsum);
   for (int w = 0; w < (tid >> 6); ++w) running += wsum[w];
@@ -172,9 +178,14 @@ __global__ __launch_bounds__(kHistThreads) void select_hist_kernel(const float *
   // range (float order = key order for non-NaN values, -0.0 == +0.0); the key itself is worked
   // out only for the members.
   constexpr int kLowBits = PASS == 1 ? 21 : 10;
-  const uint32_t lo_key = PASS == 0 ? 0u : prefix << kLowBits;
+  uint32_t lo_key = PASS == 0 ? 0u : prefix << kLowBits;
   uint32_t hi_key = PASS == 0 ? 0u : (lo_key | ((1u << kLowBits) - 1u));
   if (hi_key == 0x7fffffffu) hi_key = 0x7ffffffeu;  // the key below +-0.0's: the zeros are not in this range
+  // the bins that hold +inf / -inf reach into keys that decode to NaN, with which every compare
+  // is false: the bounds stop at the keys of the infinities
+  constexpr uint32_t kKeyPosInf = 0xff800000u, kKeyNegInf = 0x007fffffu;
+  if (hi_key > kKeyPosInf) hi_key = kKeyPosInf;
+  if (lo_key < kKeyNegInf) lo_key = kKeyNegInf;
   const float lo_f = key_to_float(lo_key), hi_f = key_to_float(hi_key);
   auto count = [&](float f) {
     if (PASS == 0) {
@@ -316,7 +327,7 @@ __global__ __launch_bounds__(kCompactThreads) void count_ranges_kernel(
 
 template <bool DIRECT>
 __global__ __launch_bounds__(kCompactThreads) void write_ranges_kernel(
-    const float *__restrict__ p, int64_t n, const State *state, int64_t wave_len,
+    const float *__restrict__ p, int64_t n, int64_t k, const State *state, int64_t wave_len,
     const uint64_t *__restrict__ wave_counts, const uint64_t *__restrict__ block_counts,
     const uint32_t *__restrict__ lists, int list_cap, uint32_t *__restrict__ ckey,
     uint32_t *__restrict__ cidx, float *__restrict__ values_out,
@@ -350,6 +361,7 @@ __global__ __launch_bounds__(kCompactThreads) void write_ranges_kernel(
   uint32_t gt_run = (uint32_t)(excl >> 31), eq_run = (uint32_t)(excl & 0x7fffffff);
 
   auto emit = [&](uint32_t pos, int64_t index, float value, uint32_t key) {
+    if (pos >= (uint32_t)k) return;  // counts that NaN priorities put out of step never leave the outputs
     if (DIRECT) {
       indices_out[pos] = index;
       if (values_out) values_out[pos] = value;
@@ -423,21 +435,24 @@ struct EmitSorted {
   const float *p;
   float *values;
   int64_t *indices;
+  uint32_t n;
   __device__ __forceinline__ void operator()(uint32_t pos, uint32_t, uint32_t index) const {
+    // index < n always holds for valid input; with NaN priorities fewer than k candidates are
+    // written and the rest of the candidate arrays is whatever the workspace held
     indices[pos] = (int64_t)index;
-    if (values) values[pos] = p[index];
+    if (values) values[pos] = index < n ? p[index] : 0.0f;
   }
 };
 
 __global__ __launch_bounds__(kBlock) void emit_kernel(const float *__restrict__ p,
                                                       const uint32_t *__restrict__ sidx, int64_t k,
-                                                      float *__restrict__ values_out,
+                                                      int64_t n, float *__restrict__ values_out,
                                                       int64_t *__restrict__ indices_out) {
   const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (j >= k) return;
   const uint32_t i = sidx[j];
   indices_out[j] = (int64_t)i;
-  if (values_out) values_out[j] = p[i];
+  if (values_out) values_out[j] = (int64_t)i < n ? p[i] : 0.0f;
 }
 
 }  // namespace
@@ -488,11 +503,11 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
                                                wave_len, wave_counts, block_counts, lists,
                                                (int)g.list_cap);
   if (direct)
-    write_ranges_kernel<true><<<cgrid, cblock, 0, st>>>(priorities, n, state, wave_len, wave_counts,
+    write_ranges_kernel<true><<<cgrid, cblock, 0, st>>>(priorities, n, k, state, wave_len, wave_counts,
                                                        block_counts, lists, (int)g.list_cap, ckey,
                                                        cidx, values_out, indices_out);
   else
-    write_ranges_kernel<false><<<cgrid, cblock, 0, st>>>(priorities, n, state, wave_len,
+    write_ranges_kernel<false><<<cgrid, cblock, 0, st>>>(priorities, n, k, state, wave_len,
                                                         wave_counts, block_counts, lists,
                                                         (int)g.list_cap, ckey, cidx, values_out,
                                                         indices_out);
@@ -505,14 +520,14 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   uint32_t *shist = reinterpret_cast<uint32_t *>(ws + l.shist);
   if (k > radix::kRankMax) {
     // radix path: the last digit's scatter writes values_out / indices_out itself
-    const EmitSorted fin{priorities, values_out, indices_out};
+    const EmitSorted fin{priorities, values_out, indices_out, (uint32_t)n};
     return radix::sort_pairs<uint32_t, uint32_t, EmitSorted>(ckey, skey, cidx, sidx, tkey, tidx, k,
                                                              0, 32, shist, st, fin);
   }
   int rc = radix::sort_pairs<uint32_t, uint32_t>(ckey, skey, cidx, sidx, tkey, tidx, k, 0, 32,
                                                  shist, st);
   if (rc) return rc;
-  emit_kernel<<<dim3((unsigned)ceil_div64(k, kBlock)), block, 0, st>>>(priorities, sidx, k,
+  emit_kernel<<<dim3((unsigned)ceil_div64(k, kBlock)), block, 0, st>>>(priorities, sidx, k, n,
                                                                       values_out, indices_out);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;

@@ -22,7 +22,20 @@ from ..dataset import SharedDataset
 from ..dtypes import CVT_DTYPES_GEAR_TO_TORCH
 from ..libgear import core as glibc
 from ..utils import get_local_node_hashed_int32
-from .basic_loader import BasicLoader
+
+
+class BasicLoader:
+    """Interface of every loader (gear/loader/basic_loader.py:4-14): a batch size, iteration,
+    and a checkpoint hook that subclasses may provide."""
+
+    def __init__(self, batch_size) -> None:
+        self._batch_size = batch_size
+
+    def __next__(self):
+        raise NotImplementedError
+
+    def checkpoint(self):
+        raise NotImplementedError
 
 
 def ensure_dataset(dataset):
@@ -130,10 +143,16 @@ class OfflineLoader(BasicLoader):
         index set is updated too (what SharedMemoryIndexServer.update is meant to do,
         src/index/server.cc:175-180).  Returns the number of updated trajectories."""
         cap = cache.capacity
-        if not hasattr(self, "_upd_idx") or self._upd_idx.numel() < 2 * cap:
+        if getattr(self, "_upd_idx", None) is None or self._upd_idx.numel() < 2 * cap:
             pin = torch.cuda.is_available()
             self._upd_idx = torch.empty(2 * cap, dtype=torch.int64, pin_memory=pin)
             self._upd_w = torch.empty(cap, dtype=torch.float32, pin_memory=pin)
+            self._upd_uploaded = None
+        # the uploads of the previous flush read these pinned buffers asynchronously: they must
+        # have left before continuous() overwrites them
+        if self._upd_uploaded is not None:
+            self._upd_uploaded.synchronize()
+            self._upd_uploaded = None
         num = cache.continuous(self._upd_idx, self._upd_w)
         if num == 0:
             return 0
@@ -149,7 +168,29 @@ class OfflineLoader(BasicLoader):
         ops.scatter(self._device_weights, didx, w.to(dev, non_blocking=True), unique_indices=True)
         ops.scatter(self._device_timesteps, didx, ts.to(dev, non_blocking=True),
                     unique_indices=True)
+        if self._upd_idx.is_pinned():
+            self._upd_uploaded = torch.cuda.Event()
+            self._upd_uploaded.record(torch.cuda.current_stream(dev))
         return num
+
+    def partition_indices(self, global_indices):
+        """indices_partitions[i][j] = the indices of rank i's slice of the batch that live in rank
+        j's shard (gear/loader/offline_loader.py:123-140).  On this build's single rank: one
+        slice holding the whole batch, one shard [0, capacity)."""
+        batch_size = global_indices.size(0)
+        slice_size = max(int(batch_size / self._dp_world), 1)
+        parts = [[None] * self._dp_world for _ in range(self._dp_world)]
+        for i in range(self._dp_world):
+            assigned = global_indices[slice_size * i:slice_size * (i + 1)]
+            for j in range(self._dp_world):
+                lo = j * self._dp_capacity
+                parts[i][j] = assigned[(lo <= assigned) & (assigned < lo + self._dp_capacity)]
+        return parts
+
+    def generate_rank_comm_order(self):
+        """Peer schedule of the shard exchange: step k talks to rank (k - dp_rank) mod world
+        (gear/loader/offline_loader.py:142-153); [0] on one rank."""
+        return [(k - self._dp_rank) % self._dp_world for k in range(self._dp_world)]
 
     @property
     def table_spec(self):

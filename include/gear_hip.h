@@ -218,8 +218,11 @@ int gear_hip_rescan_f32_f64(const float *in, double *out, int64_t n, int64_t fir
 int gear_hip_scan_f32_f32(const float *in, float *out, int64_t n, void *workspace,
                           size_t workspace_bytes, void *stream);
 
-/* Same scan over int64 weights (trajectory lengths, include/index/set.h:42), exact in int64.
- * Used for length-weighted trajectory sampling (BASELINE config 3). */
+/* Same scan over int64 weights (trajectory lengths, include/index/set.h:42), exact in int64
+ * (two's complement: weights of either sign, sums wrap like int64 additions).
+ * Used for length-weighted trajectory sampling (BASELINE config 3).
+ * Always the two-launch form, in which no workgroup waits for another; n <= 2^26 = 67 108 864,
+ * GEAR_HIP_ERANGE beyond. */
 int gear_hip_scan_i64(const int64_t *in, int64_t *out, int64_t n, void *workspace,
                       size_t workspace_bytes, void *stream);
 

@@ -323,3 +323,64 @@ def test_graph_loader_equals_eager_loader(method):
         assert torch.equal(ts_e, ts_g), "iteration %d" % it
         for a, b in zip(b_e, b_g):
             assert torch.equal(a, b), "iteration %d" % it
+
+
+@pytest.mark.parametrize("placement", ["pinned", "device"])
+def test_handler_subcopy_ignores_indices_outside_the_table(placement):
+    """handler.subcopy under the reference's own name (src/storage/pybind.cc:140-146) takes the
+    checked launch: a negative or too large trajectory index gathers nothing (its rows keep the
+    caller's zeros, as the reference's pre-zeroed batch does) instead of reading outside the
+    table; the windows with valid indices are what they were."""
+    ds, raw = _dataset(placement, seed=31)
+    handler = ds._handler
+    from gear_amd.libgear import core as glibc
+    handler.set([0], [glibc.SubscribePattern(-40, 40, glibc.SubscribePattern.PadOption.tail)])
+    idx = torch.tensor([0, -1, 47, 48, 5, 1 << 40, -(1 << 50), 13], device="cuda")
+    good = [0, 2, 4, 7]
+    lens = torch.tensor([raw["len"][i] if 0 <= i < 48 else 40 for i in idx.tolist()],
+                        device="cuda")
+    announce("handler.subcopy with indices outside the table, placement=%s" % placement)
+    for zero_fill in (False, True):
+        dst = torch.zeros((8, 40, 11), dtype=torch.float32, device="cuda") if not zero_fill \
+            else torch.full((8, 40, 11), 7.0, dtype=torch.float32, device="cuda")
+        handler.subcopy(idx, lens, lens, 0, dst, zero_fill=zero_fill)
+        torch.cuda.synchronize()
+        out = dst.cpu()
+        for row in range(8):
+            if row in good:
+                tid = int(idx[row])
+                n = raw["len"][tid]
+                assert torch.equal(out[row, :n], raw["observations"][tid])
+                assert not out[row, n:].any()
+            else:
+                assert not out[row].any()
+
+
+def test_two_cached_update_flushes_back_to_back(oracle):
+    """Two apply_cached_updates calls with no synchronisation in between reuse the same pinned
+    staging buffers: the second flush must wait for the first one's uploads.  Device state after
+    both equals the host restatement (last write wins inside a flush, later flush wins)."""
+    from gear_amd.libgear import core as glibc
+    from gear_amd.loader import OfflineLoader
+    ds, raw = _dataset("pinned", capacity=4096, T=4, seed=33)
+    loader = OfflineLoader(ds, 8, _mpu(), "TopK", PATTERNS_SHORT, timesteps_on_device=True)
+    w = ds.weights.numpy().copy()
+    ts = ds.timesteps.numpy().copy()
+    rng = np.random.default_rng(33)
+    cache = glibc.CachedRequest(4096)
+    announce("two flushes of cached updates back to back")
+    for flush in range(6):
+        for _ in range(3000):
+            i = int(rng.integers(0, 4096))
+            t = int(rng.integers(1, 5))
+            x = float(np.float32(rng.random() + 1.0 + flush))
+            cache.warr.update(i, t, x)
+            w[i], ts[i] = np.float32(x), t
+        assert loader.apply_cached_updates(cache) > 0     # no synchronize between flushes
+    torch.cuda.synchronize()
+    assert np.array_equal(loader._device_weights.cpu().numpy(), w)
+    assert np.array_equal(loader._device_timesteps.cpu().numpy(), ts)
+    assert np.array_equal(ds.weights.numpy(), w) and np.array_equal(ds.timesteps.numpy(), ts)
+
+
+PATTERNS_SHORT = [{"name": "observations", "offset": -4, "length": 4, "pad": "tail"}]

@@ -318,3 +318,37 @@ def test_split_step_index():
         assert np.array_equal(idxs.cpu().numpy(), f // T)
         assert np.array_equal(tss.cpu().numpy(), f % T)
         assert np.array_equal(lens.cpu().numpy(), f % T + 1)
+
+
+@pytest.mark.parametrize("n", [4097, 100_000, 3_000_001])
+def test_scan_i64_signed_weights_with_range_sums_of_minus_one(oracle, n, scan_variant):
+    """int64 weights of either sign whose range sums are -1 (the all-ones word): the int64 scan
+    never takes a kernel that marks unpublished sums with that word, whatever the environment
+    selects, and stays exact."""
+    from gear_amd import ops
+    rng = np.random.default_rng(n)
+    w = rng.integers(-5, 6, size=n).astype(np.int64)
+    # make every 2048-element stretch (the smallest range) sum to -1, and so every larger range
+    # of 2^k of them sum to -2^k; a second array makes the larger ranges sum to -1 as well
+    for width in (2048, 4096, 8192, 16384):
+        v = w.copy()
+        for s in range(0, n - width + 1, width):
+            v[s + width - 1] -= v[s:s + width].sum() + 1
+        announce("scan int64 signed n=%d range width %d %s" % (n, width, scan_variant))
+        got = ops.prefix_sum_i64(_dev(v)).cpu().numpy()
+        assert np.array_equal(got, np.cumsum(v))
+        assert np.array_equal(got, oracle.scan_i64(v))
+
+
+def test_scan_i64_beyond_its_limit_is_refused():
+    from gear_amd import _cabi
+    lib = _cabi.load()
+    x = torch.zeros(16, dtype=torch.int64, device="cuda")
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    n = (1 << 26) + 1
+    need = lib.gear_hip_scan_workspace_bytes(n)
+    assert need <= ws.numel()
+    import ctypes
+    rc = lib.gear_hip_scan_i64(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(x.data_ptr()), n,
+                               ctypes.c_void_p(ws.data_ptr()), ws.numel(), None)
+    assert rc == -3

@@ -57,6 +57,52 @@ def test_topk_cases(oracle):
     _check_topk(oracle, ops, ln(2_000_000), 2_500, "same size, spread out (lists)")
 
 
+def test_topk_infinite_priorities(oracle):
+    """The k-th largest priority is +inf (at least k of them), or the selection reaches down to
+    -inf (k == n): the bins of the infinities border on keys that decode to NaN."""
+    from gear_amd import ops
+    rng = np.random.default_rng(61)
+    w = (rng.lognormal(0, 1, size=200_000) ** 0.6).astype(np.float32)
+    w[rng.permutation(200_000)[:5_000]] = np.inf
+    _check_topk(oracle, ops, w, 3_000, "k-th largest is +inf")
+    _check_topk(oracle, ops, w, 5_000, "exactly k +inf")
+    _check_topk(oracle, ops, w, 5_001, "one below the +inf")
+    v = rng.normal(size=70_000).astype(np.float32)
+    v[rng.permutation(70_000)[:900]] = -np.inf
+    v[rng.permutation(70_000)[:50]] = np.inf
+    _check_topk(oracle, ops, v, 70_000, "k == n with -inf")
+    _check_topk(oracle, ops, v, 69_500, "threshold is -inf")
+    _check_topk(oracle, ops, np.full(5_000, -np.inf, np.float32), 100, "all -inf")
+    _check_topk(oracle, ops, np.full(5_000, np.inf, np.float32), 4_999, "all +inf")
+
+
+def test_topk_nan_priorities_stay_inside_the_outputs():
+    """NaN is not a valid priority and the selection is then unspecified, but nothing may be
+    written outside values_out[0:k) / indices_out[0:k)."""
+    from gear_amd import _cabi
+    import ctypes
+    lib = _cabi.load()
+    rng = np.random.default_rng(62)
+    n = 300_000
+    for frac, k in ((0.001, 4_096), (0.5, 4_096), (1.0, 4_096), (0.5, 20_000), (1.0, 20_000)):
+        w = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+        w[rng.random(n) < frac] = np.nan
+        dw = _dev(w)
+        for by_value in (0, 1):
+            vals = torch.full((k + 1024,), -7.0, dtype=torch.float32, device="cuda")
+            idx = torch.full((k + 1024,), -7, dtype=torch.int64, device="cuda")
+            ws = torch.empty(lib.gear_hip_topk_workspace_bytes(n, k), dtype=torch.uint8,
+                             device="cuda")
+            announce("topk with NaN fraction %g by_value=%d" % (frac, by_value))
+            rc = lib.gear_hip_topk_f32(ctypes.c_void_p(dw.data_ptr()), n, k, by_value,
+                                       ctypes.c_void_p(vals.data_ptr()),
+                                       ctypes.c_void_p(idx.data_ptr()),
+                                       ctypes.c_void_p(ws.data_ptr()), ws.numel(), None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            assert bool((vals[k:] == -7.0).all()) and bool((idx[k:] == -7).all())
+
+
 def test_topk_config5_size(oracle):
     """Config 5's maintenance step at full size: top-65 536 of 10 000 000 lognormal^0.6."""
     from gear_amd import ops

@@ -315,3 +315,28 @@ def test_weight_update_requests_dedupe_last_wins():
     cache.iarr.insert(2, 7, 11)
     assert cache.iarr.count == 1 and cache.iarr.index_element_view(0) == 7
     assert cache.iarr.timestep_tensor_view().tolist() == [11]
+
+
+def test_loader_partition_and_rank_order_on_one_rank():
+    """OfflineLoader.partition_indices / generate_rank_comm_order
+    (gear/loader/offline_loader.py:123-153) at a data-parallel world of 1: one slice with the
+    whole batch, one shard, peer order [0]; indices outside the shard are dropped."""
+    from gear_amd.dataset import SharedDataset
+    from gear_amd.loader import OfflineLoader
+    from gear_amd.loader.offline_loader import BasicLoader
+    from gear_amd.mpu import ModelParallelismUnit
+    tspec = TableSpec.create(trajectory_length=4, capacity=6,
+                             column_specs=[{"shape": [2], "dtype": torch.float32, "name": "obs"}])
+    ds = SharedDataset.create(tspec, key=os.getpid() + 77, placement="host")
+    for i in range(6):
+        ds[i] = (1.0, 4, [torch.full((4, 2), float(i))])
+    loader = OfflineLoader(ds, 3, ModelParallelismUnit(device="cpu"), "Uniform",
+                           [{"name": "obs", "offset": 0, "length": 4}])
+    assert isinstance(loader, BasicLoader)
+    parts = loader.partition_indices(torch.tensor([0, 5, 2, 9, -1, 3]))
+    assert len(parts) == 1 and len(parts[0]) == 1
+    assert parts[0][0].tolist() == [0, 5, 2, 3]
+    assert loader.generate_rank_comm_order() == [0]
+    gear_amd.install_as_gear()
+    from gear.loader.basic_loader import BasicLoader as B2
+    assert B2 is BasicLoader
