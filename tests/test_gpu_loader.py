@@ -384,3 +384,64 @@ def test_two_cached_update_flushes_back_to_back(oracle):
 
 
 PATTERNS_SHORT = [{"name": "observations", "offset": -4, "length": 4, "pad": "tail"}]
+
+
+@pytest.mark.parametrize("src_placement,dst_placement", [("device", "pinned"), ("pinned", "device"),
+                                                         ("device", "device")])
+def test_checkpoint_round_trip_between_placements(tmp_path, src_placement, dst_placement):
+    """SharedDataset.checkpoint / load (gear/dataset/shared_dataset.py:179-258) with the table in
+    HBM or in pinned host memory: the table pickle (src/storage/pybind.cc:178-204) reads a device
+    table back through the library, the loaded copy lands in the other placement, and both
+    datasets gather byte-identical batches.  The index state travels as the reference's PACKED
+    blob -- timesteps int64[n] directly followed by weights fp32[n] at byte 8n, not at the
+    128-byte-rounded offset the live index set uses (include/index/set.h:158-181,
+    src/index/pybind.cc:15-50)."""
+    from gear_amd.dataset import SharedDataset
+    from gear_amd.loader import OfflineLoader
+    cap = 50                                          # 8 * 50 = 400 is not a multiple of 128
+    ds, raw = _dataset(src_placement, capacity=cap, seed=41)
+    assert ds._table.placement == src_placement
+    path = tmp_path / "ckpt" / "ds.pt"
+    announce("checkpoint %s table, load as %s" % (src_placement, dst_placement))
+    ds.checkpoint(path)
+    state = ds._iset.get_state().__getstate__()
+    blob = np.asarray(state[3]).view(np.uint8)
+    assert blob.size == 8 * cap + 4 * cap
+    assert np.array_equal(blob[:8 * cap].view(np.int64), ds.timesteps.numpy())
+    assert np.array_equal(blob[8 * cap:].view(np.float32), ds.weights.numpy())
+    os.environ["GEAR_TABLE_PLACEMENT"] = dst_placement
+    try:
+        ds2 = SharedDataset().load(path, key=os.getpid() + 4100)
+    finally:
+        del os.environ["GEAR_TABLE_PLACEMENT"]
+    assert ds2._table.placement == dst_placement
+    assert torch.equal(ds2.weights, ds.weights) and torch.equal(ds2.timesteps, ds.timesteps)
+    # the table bytes, read back through the handler of each placement
+    nbytes = int(ds._table.get_table_spec().size())
+    a = torch.empty(nbytes, dtype=torch.uint8)
+    b = torch.empty(nbytes, dtype=torch.uint8)
+    ds._handler.raw(0, nbytes).copy_to(a)
+    ds2._handler.raw(0, nbytes).copy_to(b)
+    assert torch.equal(a, b) and bool(a.any())
+    # and what the gather makes of them
+    indices = torch.arange(cap, dtype=torch.long)
+    l1 = OfflineLoader(ds, 16, _mpu(), "Uniform", PATTERNS)
+    l2 = OfflineLoader(ds2, 16, _mpu(), "Uniform", PATTERNS)
+    b1 = l1.exposed_fused_iterate(indices)
+    b2 = l2.exposed_fused_iterate(indices)
+    torch.cuda.synchronize()
+    for x, y in zip(b1, b2):
+        assert torch.equal(x, y)
+    for tid in range(cap):
+        n = raw["len"][tid]
+        assert torch.equal(b2[0][tid, :n].cpu(), raw["observations"][tid])
+    # same sampler seed, same batches from both
+    w1 = OfflineLoader(ds, 8, _mpu(), "Weighted", PATTERNS)
+    w2 = OfflineLoader(ds2, 8, _mpu(), "Weighted", PATTERNS)
+    for _ in range(3):
+        t1, x1 = next(w1)
+        t2, x2 = next(w2)
+        torch.cuda.synchronize()
+        assert torch.equal(t1, t2)
+        for x, y in zip(x1, x2):
+            assert torch.equal(x, y)
