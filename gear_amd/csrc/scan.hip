@@ -3,19 +3,24 @@
 // Three kernels share the inner scan (each thread scans inside its 16-byte input vectors, row sums
 // go through a DPP wave scan, wave totals meet in LDS, results leave through LDS so that every store
 // instruction writes whole lines):
-//  * default, up to 8192 ranges (n <= 134 M fp32): two launches.  range_sum_kernel writes the sum
-//    of every range; scan_ranges_kernel<TWO = true> re-reads its range (now in L2 / MALL), adds
-//    the sums of all earlier ranges in a fixed order and writes the prefix.  No workgroup waits for
-//    another one.  On this multi-XCD part that is faster than the one-pass kernels: a ticket per
-//    workgroup on one address costs ~19 ns each across the XCDs, and every agent-scope round trip
-//    of a look-back 1-2 us.
-//  * GEAR_HIP_SCAN_SINGLE_PASS=1: scan_ranges_kernel<TWO = false>, one pass over the data.  Tile
-//    numbers are handed out by an atomic ticket in launch order (every awaited predecessor is
-//    already running); a workgroup publishes the sum of its range in one agent-scope 64-bit store
-//    (kEmpty = not published, so no fence pairs) and sums ALL earlier ranges' words.
-//  * beyond that (and beyond 2048 ranges in the single-pass mode): scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone,
+//  * chained single pass, up to 2048 ranges: scan_ranges_kernel<CHAINED = true>.  A workgroup
+//    keeps its range in registers, publishes the range's sum and adds the sums of ALL earlier
+//    ranges (fixed order: bit-reproducible), then writes the prefix: the input is read once.
+//    Range r belongs to workgroup r (no ticket).  A published sum travels as three 64-bit words
+//    that each carry 42 bits of the call's tag next to 21 or 22 bits of payload, so a word is valid
+//    on its own: no fence, no flag, nothing to clear before a call (a host counter hands every
+//    call a fresh tag; what an earlier call or an uninitialised workspace left never matches).
+//    The wait for a predecessor is bounded: when it runs out, the workgroup sums that
+//    predecessor's range itself, with the same reduction tree, so no kernel can spin forever and
+//    the result does not change.
+//  * two launches, up to 8192 ranges (n <= 134 M fp32): range_sum_kernel writes the sum of every
+//    range; scan_ranges_kernel<CHAINED = false> re-reads its range (now in L2 / MALL), adds the
+//    sums of all earlier ranges and writes the prefix.  No workgroup waits for another one.  Used
+//    for long inputs, under stream capture (a captured launch would replay its tag) and for the
+//    incremental rescan of a suffix.
+//  * beyond that: scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone,
 //    incl[t] = sum of tiles 0..t; wave 0 looks back 64 predecessors at a time, ballots pick the
-//    nearest published inclusive value).
+//    nearest published inclusive value; tile numbers come from an atomic ticket).
 #include <atomic>
 #include <type_traits>
 
@@ -230,74 +235,107 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
 }
 
 // ---- range variant -------------------------------------------------------------------------------
-// For up to kMaxRanges workgroups the look-back chain is not needed at all: a workgroup owns NR
-// rows of 256 vectors kept in registers, publishes the sum of its range as soon as it has loaded
-// it, and takes its exclusive prefix as the sum of ALL earlier ranges' aggregates (each thread
-// polls its share of them, fixed summation order).  Nobody waits for an inclusive value, so there
-// is no serial chain across the XCDs, and the result is bit-reproducible from run to run.
-constexpr int kMaxRanges = 2048;     // single-pass variant: every thread polls 8 range sums
+// A workgroup owns NR rows of 256 vectors kept in registers and takes its exclusive prefix as the
+// sum of ALL earlier ranges' sums (each thread adds its share of them, fixed summation order).
+// Nobody waits for an inclusive value, so there is no serial chain across the XCDs, and the result
+// is bit-reproducible from run to run.
+constexpr int kMaxRanges = 2048;     // chained: every thread polls up to 8 range sums
 constexpr int kMaxRangesTwo = 8192;  // two launches: every thread adds up to 32 range sums
 
-// Sum of every range, one workgroup per range: the first launch of the two-launch variant, in
-// which the scan launch below finds all aggregates ready (no ticket, no publishing, no polling).
+// A range sum in flight between workgroups of one launch: three self-validating words.
+constexpr int kTagBits = 42;
+constexpr uint64_t kTagMask = (1ull << kTagBits) - 1ull;
+struct Slot {
+  uint64_t w[3];
+};
+__device__ __forceinline__ void publish(Slot *s, uint64_t tag, uint64_t v) {
+  store_agent(&s->w[0], (tag << 22) | (v & 0x3fffffull));
+  store_agent(&s->w[1], (tag << 22) | ((v >> 22) & 0x1fffffull));
+  store_agent(&s->w[2], (tag << 22) | (v >> 43));
+}
+__device__ __forceinline__ bool try_read(const Slot *s, uint64_t tag, uint64_t *v) {
+  const uint64_t a = load_agent(&s->w[0]), b = load_agent(&s->w[1]), c = load_agent(&s->w[2]);
+  *v = (a & 0x3fffffull) | ((b & 0x1fffffull) << 22) | ((c & 0x1fffffull) << 43);
+  return (a >> 22) == tag && (b >> 22) == tag && (c >> 22) == tag;
+}
+
+// The sum of one range with the reduction tree every kernel here uses for it (thread: rows in
+// order, vector elements in order; wave: DPP tree; workgroup: (w0 + w1) + (w2 + w3)), returned to
+// every thread.  `red` is LDS for the four wave sums; the caller separates calls with a barrier.
 template <typename In, typename Acc, int VE, int NR>
-__global__ __launch_bounds__(kBlock) void range_sum_kernel(const In *__restrict__ in, int64_t n,
-                                                           uint64_t *__restrict__ aggr,
-                                                           int64_t first_range) {
+__device__ __forceinline__ Acc range_total(const In *__restrict__ in, int64_t n, int64_t range,
+                                           Acc *red) {
   constexpr int kElems = NR * kBlock * VE;
-  constexpr int kWaves = kBlock / kWave;
   typedef typename InVec<In, VE>::type in_vec;
-  __shared__ Acc red[kWaves];
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-  const int64_t range = first_range + blockIdx.x;
   const int64_t base = range * kElems;
-  In raw[NR][VE];
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
-    if (e0 + VE <= n) {
-      const in_vec v = *reinterpret_cast<const in_vec *>(in + e0);
-#pragma unroll
-      for (int j = 0; j < VE; ++j) raw[r][j] = v[j];
-    } else {
-#pragma unroll
-      for (int j = 0; j < VE; ++j) raw[r][j] = (e0 + j < n) ? in[e0 + j] : (In)0;
-    }
-  }
   Acc tsum = (Acc)0;
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
-    Acc a = (Acc)raw[r][0];
+    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
+    In raw[VE];
+    if (e0 + VE <= n) {
+      const in_vec v = *reinterpret_cast<const in_vec *>(in + e0);
 #pragma unroll
-    for (int j = 1; j < VE; ++j) a += (Acc)raw[r][j];
+      for (int j = 0; j < VE; ++j) raw[j] = v[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < VE; ++j) raw[j] = (e0 + j < n) ? in[e0 + j] : (In)0;
+    }
+    Acc a = (Acc)raw[0];
+#pragma unroll
+    for (int j = 1; j < VE; ++j) a += (Acc)raw[j];
     tsum += a;
   }
   const Acc w = wave_sum(tsum);
   if (lane == 0) red[wave] = w;
   __syncthreads();
-  if (tid == 0) aggr[range] = Bits<Acc>::to((red[0] + red[1]) + (red[2] + red[3]));
+  const Acc total = (red[0] + red[1]) + (red[2] + red[3]);
+  __syncthreads();
+  return total;
 }
 
-template <typename In, typename Acc, typename Out, int VE, int NR, bool TWO>
+// Sum of every range, one workgroup per range: the first launch of the two-launch variant, in
+// which the scan launch below finds all sums ready (no publishing, no polling).
+template <typename In, typename Acc, int VE, int NR>
+__global__ __launch_bounds__(kBlock) void range_sum_kernel(const In *__restrict__ in, int64_t n,
+                                                           uint64_t *__restrict__ sums,
+                                                           int64_t first_range) {
+  __shared__ Acc red[kBlock / kWave];
+  const int64_t range = first_range + blockIdx.x;
+  const Acc total = range_total<In, Acc, VE, NR>(in, n, range, red);
+  if (threadIdx.x == 0) sums[range] = Bits<Acc>::to(total);
+}
+
+// sums[r]   plain range sums (kept between calls: the incremental rescan reuses the ones before
+//           its first range)
+// slots[r]  CHAINED only: the same sums as tagged words, for the workgroups of this launch
+// spin_limit  CHAINED only: polls of a missing predecessor before the workgroup sums that range
+//           itself
+template <typename In, typename Acc, typename Out, int VE, int NR, bool CHAINED>
 __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restrict__ in,
                                                              Out *__restrict__ out, int64_t n,
-                                                             uint32_t *ticket, uint64_t *aggr,
-                                                             int64_t first_range) {
+                                                             uint64_t *__restrict__ sums,
+                                                             Slot *__restrict__ slots,
+                                                             int64_t first_range, uint64_t tag,
+                                                             int spin_limit) {
   constexpr int kElems = NR * kBlock * VE;
   constexpr int kWaves = kBlock / kWave;
   typedef typename InVec<In, VE>::type in_vec;
   __shared__ Acc wtot[NR][kWaves];
   __shared__ Out stage[kWaves][kWave * VE];
   __shared__ Acc red[kWaves];
-  __shared__ uint32_t s_tile;
+  __shared__ int s_missing;
+  __shared__ uint16_t s_queue[CHAINED ? kMaxRanges : 1];
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-  if (!TWO) {
-    if (tid == 0) s_tile = atomicAdd(ticket, 1u);
+  const int64_t tile = first_range + (int64_t)blockIdx.x;
+  const int64_t base = tile * kElems;
+
+  if (CHAINED) {
+    if (tid == 0) s_missing = 0;
     __syncthreads();
   }
-  const int64_t tile = TWO ? first_range + (int64_t)blockIdx.x : (int64_t)s_tile;
-  const int64_t base = tile * kElems;
 
   In raw[NR][VE];
   Acc s[NR];
@@ -322,12 +360,16 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
     s[r] = a;
     tsum += a;
   }
-  // the range's aggregate goes out before the detailed scan
-  if (!TWO) {
+  // the range's sum goes out before the detailed scan
+  if (CHAINED) {
     const Acc w = wave_sum(tsum);
     if (lane == 0) red[wave] = w;
     __syncthreads();
-    if (tid == 0) store_agent(&aggr[tile], Bits<Acc>::to((red[0] + red[1]) + (red[2] + red[3])));
+    if (tid == 0) {
+      const uint64_t bits = Bits<Acc>::to((red[0] + red[1]) + (red[2] + red[3]));
+      publish(&slots[tile], tag, bits);
+      sums[tile] = bits;
+    }
   }
   Acc wexcl[NR];
 #pragma unroll
@@ -336,27 +378,52 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
     wexcl[r] = wave_shift_up1(inc);
     if (lane == kWave - 1) wtot[r][wave] = inc;
   }
-  // sum of every earlier range (thread t takes ranges t, t+256, ...)
-  // all of a thread's polls are issued together; only the ones not yet published are repeated
-  constexpr int kPolls = (TWO ? kMaxRangesTwo : kMaxRanges) / kBlock;
+  // sum of every earlier range (thread t takes ranges t, t+256, ...): the ones before this
+  // launch's first range are plain words from an earlier call, the others are published by the
+  // workgroups of this launch.  All of a thread's polls are issued together; only the ones not
+  // yet published are repeated.
+  constexpr int kPolls = (CHAINED ? kMaxRanges : kMaxRangesTwo) / kBlock;
   uint64_t pv[kPolls];
+  bool have[kPolls];
 #pragma unroll
   for (int i = 0; i < kPolls; ++i) {
     const int64_t j = tid + (int64_t)i * kBlock;
-    pv[i] = j < tile ? (TWO ? aggr[j] : load_agent(&aggr[j])) : 0ull;
-  }
-  bool pending = !TWO;
-  while (pending) {
-    pending = false;
-#pragma unroll
-    for (int i = 0; i < kPolls; ++i) {
-      const int64_t j = tid + (int64_t)i * kBlock;
-      if (j < tile && pv[i] == kEmpty) {
-        pv[i] = load_agent(&aggr[j]);
-        pending |= pv[i] == kEmpty;
-      }
+    pv[i] = 0ull;
+    have[i] = true;
+    if (j < tile) {
+      if (!CHAINED || j < first_range)
+        pv[i] = sums[j];
+      else
+        have[i] = try_read(&slots[j], tag, &pv[i]);
     }
-    if (pending) __builtin_amdgcn_s_sleep(1);
+  }
+  if (CHAINED) {
+    bool pending = true;
+    for (int spin = 0; pending && spin < spin_limit; ++spin) {
+      pending = false;
+#pragma unroll
+      for (int i = 0; i < kPolls; ++i) {
+        if (!have[i]) {
+          have[i] = try_read(&slots[tid + (int64_t)i * kBlock], tag, &pv[i]);
+          pending |= !have[i];
+        }
+      }
+      if (pending) __builtin_amdgcn_s_sleep(1);
+    }
+    // Whatever is still missing after the bounded wait is summed here, from the input, with the
+    // tree its own workgroup uses: same bits, and the kernel ends whatever the others do.
+#pragma unroll
+    for (int i = 0; i < kPolls; ++i)
+      if (!have[i]) s_queue[atomicAdd(&s_missing, 1)] = (uint16_t)(tid + i * kBlock);
+    __syncthreads();
+    const int missing = s_missing;
+    for (int q = 0; q < missing; ++q) {
+      const int j = s_queue[q];
+      const Acc total = range_total<In, Acc, VE, NR>(in, n, j, red);
+#pragma unroll
+      for (int i = 0; i < kPolls; ++i)
+        if (j == tid + i * kBlock) pv[i] = Bits<Acc>::to(total);
+    }
   }
   Acc part = (Acc)0;
 #pragma unroll
@@ -429,36 +496,44 @@ __global__ __launch_bounds__(kBlock) void sum_final_kernel(const double *partial
 
 int64_t scan_tiles(int64_t n, int tile_elems) { return n <= 0 ? 0 : ceil_div64(n, tile_elems); }
 
-// the workspace is sized for the smaller tile (int64: 2048 elements) so both scans fit
+// Workspace: 256-byte header (the look-back kernel's ticket), then per smallest range (2048
+// elements, so that both element types fit) one 8-byte plain sum and one 24-byte tagged slot.
+// The look-back kernel lays its two words per 4096-element tile over the same bytes.
 size_t scan_ws_bytes(int64_t n) {
   const int64_t tiles = scan_tiles(n, kRows * kBlock * 2);
-  return kHeaderBytes + align_up((size_t)tiles * 16, 256);
+  return kHeaderBytes + align_up((size_t)tiles * (8 + sizeof(Slot)), 256);
 }
 
-// first_changed > 0 (two-launch variant only): the range sums of the ranges before the one that
-// holds element first_changed are still in the workspace from the last scan of this array, and
-// `out` still holds the prefix up to there; only the later ranges are summed and scanned again.
+// every chained launch of the process gets a tag of its own
+std::atomic<uint64_t> g_scan_epoch{1};
+
+enum class Mode { kAuto, kTwoLaunch, kChained };
+
+// first_changed > 0: the sums of the ranges before the one that holds element first_changed are
+// still in the workspace from the last scan of this array, and `out` still holds the prefix up to
+// there; only the later ranges are summed and scanned again.
 template <typename In, typename Acc, typename Out, int VE, int NR>
-int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, bool single_pass,
+int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, bool chained,
                   int64_t first_changed) {
   const int64_t range_elems = (int64_t)NR * kBlock * VE;
   const int64_t ranges = ceil_div64(n, range_elems);
-  uint32_t *ticket = static_cast<uint32_t *>(ws);
-  uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
-  if (!single_pass) {
-    const int64_t first = first_changed > 0 ? first_changed / range_elems : 0;
-    const dim3 grid((unsigned)(ranges - first)), block(kBlock);
-    range_sum_kernel<In, Acc, VE, NR><<<grid, block, 0, st>>>(in, n, aggr, first);
-    scan_ranges_kernel<In, Acc, Out, VE, NR, true><<<grid, block, 0, st>>>(in, out, n, ticket, aggr,
-                                                                          first);
+  const int64_t max_ranges = scan_tiles(n, kRows * kBlock * 2);
+  uint64_t *sums = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
+  Slot *slots = reinterpret_cast<Slot *>(sums + max_ranges);
+  const int64_t first = first_changed > 0 ? first_changed / range_elems : 0;
+  const dim3 grid((unsigned)(ranges - first)), block(kBlock);
+  if (!chained) {
+    range_sum_kernel<In, Acc, VE, NR><<<grid, block, 0, st>>>(in, n, sums, first);
+    scan_ranges_kernel<In, Acc, Out, VE, NR, false><<<grid, block, 0, st>>>(in, out, n, sums, slots,
+                                                                           first, 0ull, 0);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
-  scan_init_kernel<<<dim3((unsigned)ceil_div64(ranges, kBlock)), dim3(kBlock), 0, st>>>(ticket, aggr,
-                                                                                      ranges);
-  GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  scan_ranges_kernel<In, Acc, Out, VE, NR, false><<<dim3((unsigned)ranges), dim3(kBlock), 0, st>>>(
-      in, out, n, ticket, aggr, 0);
+  uint64_t tag = g_scan_epoch.fetch_add(1, std::memory_order_relaxed) & kTagMask;
+  if (tag == 0) tag = g_scan_epoch.fetch_add(1, std::memory_order_relaxed) & kTagMask;
+  const int spin_limit = env_int("GEAR_HIP_SCAN_SPIN_LIMIT", 1 << 14);
+  scan_ranges_kernel<In, Acc, Out, VE, NR, true><<<grid, block, 0, st>>>(in, out, n, sums, slots,
+                                                                        first, tag, spin_limit);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
@@ -475,25 +550,35 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
       (reinterpret_cast<uintptr_t>(out) & 15))
     return GEAR_HIP_EALIGN;
   const int64_t row = (int64_t)kBlock * VE;
-  // Up to 8192 ranges of 2, 4, 8 or 16 rows of 256 vectors.  Default: two launches (range sums,
-  // then the scan with every aggregate ready).  GEAR_HIP_SCAN_SINGLE_PASS=1 selects the one-pass
-  // kernel with tickets and published aggregates instead (larger ranges, so that all workgroups
-  // are resident together).
-  // The kernels in which a workgroup waits for another one mark "not published yet" with the
-  // word kEmpty, which no fp64 sum of fp32 values can equal but an int64 sum can (-1): int64
-  // scans therefore always take the two launches, in which nobody waits, and stop at their limit.
-  constexpr bool kMayWait = std::is_same<Acc, double>::value;
-  const bool single_pass = kMayWait && env_int("GEAR_HIP_SCAN_SINGLE_PASS", 0) != 0;
-  const int64_t cap = single_pass ? 1024 : kMaxRanges;  // the largest ranges may be up to 8192
-  if (!single_pass && ceil_div64(n, 2 * row) <= cap)
-    return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, single_pass, first_changed);
-  if (ceil_div64(n, 4 * row) <= cap)
-    return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, single_pass, first_changed);
-  if (ceil_div64(n, 8 * row) <= cap)
-    return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, single_pass, first_changed);
-  if (ceil_div64(n, 16 * row) <= (single_pass ? kMaxRanges : kMaxRangesTwo))
-    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, single_pass, first_changed);
-  if (!kMayWait) return GEAR_HIP_ERANGE;
+  // GEAR_HIP_SCAN_SINGLE_PASS: 1 = the chained kernel wherever it applies, 0 = never; unset = the
+  // chained kernel for full scans, two launches for the rescan of a suffix.  A launch that is
+  // being captured into a graph would replay its tag, so it takes the two launches.
+  const int forced = env_int("GEAR_HIP_SCAN_SINGLE_PASS", -1);
+  bool chained = forced < 0 ? first_changed <= 0 : forced != 0;
+  if (chained) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) {
+      (void)hipGetLastError();
+      cap = hipStreamCaptureStatusActive;
+    }
+    if (cap != hipStreamCaptureStatusNone) chained = false;
+  }
+  // Ranges of 2, 4 or 8 rows of 256 vectors: the smallest that leave at most 512 ranges, else 8
+  // rows up to 2048 ranges (a workgroup adds up ALL earlier sums, so the chained kernel pays for
+  // the range count squared; 16 rows need 256 registers and run slower than twice 8).  Both
+  // variants cut the input the same way, so a rescan finds the sums of the last full scan.
+  // Beyond 2048 ranges of 8 rows: two launches with up to 8192 ranges of 16 rows.
+  if (ceil_div64(n, 2 * row) <= 512)
+    return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, chained, first_changed);
+  if (ceil_div64(n, 4 * row) <= 512)
+    return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, chained, first_changed);
+  if (ceil_div64(n, 8 * row) <= kMaxRanges)
+    return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, chained, first_changed);
+  if (ceil_div64(n, 16 * row) <= kMaxRangesTwo)
+    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, false, first_changed);
+  // The look-back kernel marks "not published yet" with the word kEmpty, which no fp64 sum of
+  // fp32 values can equal but an int64 sum can (-1): int64 scans stop at the two-launch limit.
+  if (!std::is_same<Acc, double>::value) return GEAR_HIP_ERANGE;
   const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
   uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
@@ -531,7 +616,8 @@ namespace gearhip {
 namespace {
 
 constexpr int64_t kStaticMaxN = 1ll << 27;  // 134 217 728 priorities
-constexpr size_t kStaticBytes = kHeaderBytes + (size_t)(kStaticMaxN / (kRows * kBlock * 2)) * 16;
+constexpr size_t kStaticBytes =
+    kHeaderBytes + (size_t)(kStaticMaxN / (kRows * kBlock * 2)) * (8 + sizeof(Slot));
 static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticBytes];
 
 constexpr int kMaxDevices = 64;

@@ -177,7 +177,11 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
 
 /* Inclusive prefix sum of fp32 priorities accumulated and written in fp64:
  *     out[i] = sum_{j<=i} (double) in[j]
- * Two-launch range scan (or the single-pass kernels, see GEAR_HIP_SCAN_SINGLE_PASS).  Replaces
+ * One pass over the input for up to 2048 ranges (n <= 33.5 M): every workgroup publishes the sum
+ * of its range and adds the sums of all earlier ranges, with a bounded wait (a workgroup that
+ * waited too long sums the missing range itself: same bits, no kernel can hang).  Two launches
+ * (range sums, then the scan) beyond that, for a stream under graph capture, and with
+ * GEAR_HIP_SCAN_SINGLE_PASS=0.  The result is bit-identical in all cases.  Replaces
  * gear::cuda::launch_prefix_sum /
  * one_dimension_prefix_sum (src/cuda/one_dim_prefix_sum.cu:125-273; libgear.core.prefix_sum,
  * :276-278), which is fp32 and only correct for one block.
@@ -191,7 +195,7 @@ int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspa
 /* gear_hip_scan_f32_f64 for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses with a frozen memory pool.  It has no counterpart in
  * the reference.  The range sums that the other entry point keeps in the caller's workspace live
- * in a static device array inside the library (about 1 MiB per GPU, held until the process ends);
+ * in a static device array inside the library (about 2 MiB per GPU, held until the process ends);
  * the call allocates and frees nothing.  Same result, bit for bit, as gear_hip_scan_f32_f64.
  * n <= gear_hip_scan_static_max_n() (2^27 = 134 217 728), else GEAR_HIP_ERANGE.
  * The array's address is looked up once per device, by gear_hip_set_device or by the first call
@@ -207,8 +211,7 @@ int gear_hip_scan_f32_f64_static(const float *in, double *out, int64_t n, void *
  * with the same n, and since then only in[first_changed .. n) changed.  Then out[i] is
  * recomputed from the start of the range that holds first_changed onwards, reusing the range sums
  * kept in the workspace; the result is bit-identical to a full gear_hip_scan_f32_f64.
- * first_changed >= n: nothing to do; first_changed = 0, n > 134 M or
- * GEAR_HIP_SCAN_SINGLE_PASS=1: a full scan. */
+ * first_changed >= n: nothing to do; first_changed = 0 or n > 134 M: a full scan. */
 int gear_hip_rescan_f32_f64(const float *in, double *out, int64_t n, int64_t first_changed,
                             void *workspace, size_t workspace_bytes, void *stream);
 
@@ -221,8 +224,8 @@ int gear_hip_scan_f32_f32(const float *in, float *out, int64_t n, void *workspac
 /* Same scan over int64 weights (trajectory lengths, include/index/set.h:42), exact in int64
  * (two's complement: weights of either sign, sums wrap like int64 additions).
  * Used for length-weighted trajectory sampling (BASELINE config 3).
- * Always the two-launch form, in which no workgroup waits for another; n <= 2^26 = 67 108 864,
- * GEAR_HIP_ERANGE beyond. */
+ * n <= 2^26 = 67 108 864, GEAR_HIP_ERANGE beyond (the kernel for longer inputs marks unpublished
+ * sums with a word that an int64 sum can equal). */
 int gear_hip_scan_i64(const int64_t *in, int64_t *out, int64_t n, void *workspace,
                       size_t workspace_bytes, void *stream);
 

@@ -344,11 +344,72 @@ def test_scan_i64_beyond_its_limit_is_refused():
     from gear_amd import _cabi
     lib = _cabi.load()
     x = torch.zeros(16, dtype=torch.int64, device="cuda")
-    ws = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
     n = (1 << 26) + 1
-    need = lib.gear_hip_scan_workspace_bytes(n)
-    assert need <= ws.numel()
+    ws = torch.zeros(lib.gear_hip_scan_workspace_bytes(n), dtype=torch.uint8, device="cuda")
     import ctypes
     rc = lib.gear_hip_scan_i64(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(x.data_ptr()), n,
                                ctypes.c_void_p(ws.data_ptr()), ws.numel(), None)
     assert rc == -3
+
+
+@pytest.mark.parametrize("n", [4097, 1_000_000, 3_000_001])
+def test_chained_scan_with_no_patience_sums_the_missing_ranges_itself(oracle, n):
+    """The chained kernel waits a bounded number of polls for an earlier range's sum and then sums
+    that range itself.  With a limit of 0 polls (forced from the host) every workgroup takes
+    that path for whatever is not published yet: the kernel ends and the prefix is bit-identical
+    to the two-launch result, for fp64 and int64."""
+    from gear_amd import ops
+    rng = np.random.default_rng(n)
+    p = _priorities(n, 12)
+    w = rng.integers(-3, 1000, size=n).astype(np.int64)
+    dp, dw = _dev(p), _dev(w)
+    old = {k: os.environ.get(k) for k in ("GEAR_HIP_SCAN_SINGLE_PASS", "GEAR_HIP_SCAN_SPIN_LIMIT")}
+    try:
+        os.environ["GEAR_HIP_SCAN_SINGLE_PASS"] = "0"
+        ref = ops.prefix_sum(dp).clone()
+        ref_i = ops.prefix_sum_i64(dw).clone()
+        os.environ["GEAR_HIP_SCAN_SINGLE_PASS"] = "1"
+        os.environ["GEAR_HIP_SCAN_SPIN_LIMIT"] = "0"
+        announce("chained scan, spin limit 0, n=%d" % n)
+        got = ops.prefix_sum(dp).clone()
+        got_i = ops.prefix_sum_i64(dw).clone()
+        os.environ["GEAR_HIP_SCAN_SPIN_LIMIT"] = "3"
+        got3 = ops.prefix_sum(dp).clone()
+        torch.cuda.synchronize()
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    assert torch.equal(got, ref) and torch.equal(got3, ref)
+    assert torch.equal(got_i, ref_i)
+    assert np.array_equal(got_i.cpu().numpy(), np.cumsum(w))
+
+
+def test_scan_under_graph_capture_replays_correctly(oracle):
+    """A captured scan must not bake a one-time tag into the graph: every replay (with changed
+    priorities in between) equals the eager result."""
+    from gear_amd import ops
+    n = 300_000
+    rng = np.random.default_rng(9)
+    dp = _dev(_priorities(n, 9))
+    out = torch.empty(n, dtype=torch.float64, device="cuda")
+    ops.prefix_sum(dp, out=out)                      # warm-up: workspace exists before capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.prefix_sum(dp, out=out)                  # workspace of the capture stream
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g, stream=side):
+        ops.prefix_sum(dp, out=out)
+    for it in range(4):
+        dp.copy_(_dev(_priorities(n, 100 + it)))
+        announce("graph replay %d of a captured scan" % it)
+        g.replay()
+        torch.cuda.synchronize()
+        eager = ops.prefix_sum(dp)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), it
