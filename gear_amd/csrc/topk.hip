@@ -1,37 +1,94 @@
-// Top-k of fp32 priorities by radix select + ordered compaction + radix sort, gfx950.
+// Top-k of fp32 priorities by radix select + ordered compaction + segmented ordering, gfx950.
 //
-// fp32 priorities map to order-preserving uint32 keys.  Three histogram passes (11 + 11 + 10
-// bits, LDS histograms, the consuming launch picks the bin) find the key T of the k-th largest
-// priority and how many entries equal to T are still needed.  An ordered compaction in two
-// launches writes the selected entries in index order: every entry above T, and the first need_eq
-// entries equal to T -- ties go to the smaller index.  The count launch also lists every wave's
-// candidates (entries >= T), so the write launch touches only those; where the maxima are
-// clustered a list overflows and the write launch re-reads the priorities instead.  For value
-// order the k candidates then go through the stable LSD radix sort on the inverted key.
-// The streaming loops are sensitive to their instruction count (a launch that reads 40 MB spends
-// as long issuing ~10 instructions per element as waiting for memory), so they compare floats
-// (one instruction, same order as the keys for non-NaN values) wherever a key is not needed.
+// fp32 priorities map to order-preserving uint32 keys, selected top-down in three levels: 16384
+// level-0 bins, then up to 11 and up to 10 bits inside the picked bin.  The launches of one call:
+//   prep      one workgroup draws 2048 samples and lays out the level-0 bins around them (coarse
+//             below the bin that safely lies under the k-th largest priority -- the hint --, fine
+//             from there to the largest sample, the rest above); the others clear the histograms.
+//   level 0   ONE read of the priorities: level-0 histogram (LDS, flushed with atomics) and, per
+//             wave, a list of every candidate (key | index) at or above the hint, in index order.
+//   level 1   picks the level-0 bin that holds the k-th largest key; histogram of the top bits
+//             inside that bin over its members;   level 2   the same for the remaining bits.
+//   count     picks the last digit: threshold key T and the number of entries equal to T still
+//             needed; counts (greater, equal) per wave and workgroup.
+//   write     sums the counts of the waves before it and places the selected entries in index
+//             order: every entry above T and the first `need` entries equal to T (ties go to the
+//             smaller index).
+// Levels 1, 2, count and write walk the candidate lists (about 2 % of the input) when the hint
+// held and no list overflowed; otherwise each of them streams the priorities again (count then
+// rebuilds the lists with the exact threshold, write re-reads if those overflow too).  The hint
+// only decides which of the two it is, never the result.
+// Value order (k <= 131072): write leaves the selection as (key, index, segment) in index order
+// and puts the entries equal to T straight at the tail of the output; the level-0 histogram says
+// where every bin starts in value order, bins that start in the same stretch of output places
+// form the segment of one workgroup of a last launch, which collects its entries, sorts them
+// (most-significant-digit radix sort in LDS) and writes its stretch of values and indices.
+// Larger k take the stable LSD radix sort on the inverted key.
+// The streaming loops are sensitive to their instruction count, so they compare floats (one
+// instruction, same order as the keys for non-NaN values) wherever a key is not needed.
 #include "radix_sort.hpp"
 
 namespace gearhip {
 namespace {
 
-constexpr int kBlock = 256;
-constexpr int kMaxRanges = 2048;  // workgroups of the compaction launches
-constexpr int kCompactThreads = 512;  // threads of a compaction workgroup (256: +2.5 us at n = 1e7)
-constexpr int kWavesPerBlock = kCompactThreads / kWave;
-constexpr int kHistBins = 2048;
-// Histogram launches: one 1024-thread workgroup per CU.  Fewer, fatter workgroups mean fewer
-// flush atomics per bin and fewer workgroups that pick the previous bin (measured at n = 1e7:
-// 512 x 256 threads 60.8 us for the whole top-k, 256 x 512 56.0, 512 x 1024 54.9, 256 x 1024 53.1).
-constexpr int kMaxHistBlocks = 256;
-constexpr int kHistThreads = 1024;
+constexpr int kThreads = 1024;               // every kernel of the selection
+constexpr int kWavesPerBlock = kThreads / kWave;
+constexpr int kMaxBlocks = 256;              // one workgroup per CU
+constexpr int kBins0 = 16384;  // level-0 bins
+constexpr int kBinsR = 2048;   // bins of a refinement level (up to 11 bits)
+constexpr int kUniformShift = 18;  // level-0 bins without a sample: the top 14 bits of the key
+// with a sample: keys below the hint at 12 bits, a middle stretch up to the sample's top in up to
+// kMidBins bins of its own resolution, the rest above
+constexpr int kLowShift = 20, kMidBins = 10240, kMidBinsCoarse = 256;
+constexpr int kSamples = 2048;  // two per thread of one workgroup: more would be bound by the misses one CU can have in flight
+constexpr uint32_t kNoLists = 0xffffffffu;   // hint_bin: level 0 writes no candidate lists
+constexpr int64_t kBucketMaxK = 131072;      // value order by buckets up to this k
+constexpr int kSortThreads = 1024;           // segment sort workgroup
+constexpr int kSmallGroup = 256;             // groups up to this size are ranked directly
+constexpr int kNoSegment = 255;              // segment id of an entry that no sort workgroup takes
+
+// Level-0 bins: three stretches of keys with a resolution each, so that the stretch in which the
+// selection ends -- known roughly from the sample -- is cut finely (a bin holds few entries: the
+// later levels and the value-order sort then have little to do per bin) while 16384 bins still
+// cover every key.  Without a sample: one stretch, bin = key >> kUniformShift.
+struct BinMap {
+  uint32_t uniform;  // 1: no sample
+  uint32_t a_end;    // keys below:              bin = key >> kLowShift
+  uint32_t b_last;   // a_end <= key <= b_last:  bin = nb0 + ((key - a_end) >> b_shift)
+  uint32_t nb0, nc0;  // first bin of the middle / of the top stretch
+  uint32_t b_shift, c_shift;  // keys above b_last: bin = nc0 + ((key - b_last - 1) >> c_shift)
+};
+
+__device__ __forceinline__ uint32_t bin_of(const BinMap &m, uint32_t key) {
+  if (m.uniform) return key >> kUniformShift;
+  uint32_t bin = key >> kLowShift;
+  if (key >= m.a_end) {  // about one key in a hundred
+    bin = key <= m.b_last ? m.nb0 + ((key - m.a_end) >> m.b_shift)
+                          : m.nc0 + ((key - m.b_last - 1u) >> m.c_shift);
+  }
+  return bin;
+}
+// smallest key of a bin; for one past the last bin of the map the result wraps to 0
+__device__ __forceinline__ uint32_t bin_lo_key(const BinMap &m, uint32_t bin) {
+  if (m.uniform) return bin << kUniformShift;
+  if (bin < m.nb0) return bin << kLowShift;
+  if (bin < m.nc0) return m.a_end + ((bin - m.nb0) << m.b_shift);
+  return m.b_last + 1u + ((bin - m.nc0) << m.c_shift);
+}
+__device__ __forceinline__ uint32_t bin_hi_key(const BinMap &m, uint32_t bin) {
+  return bin_lo_key(m, bin + 1u) - 1u;
+}
 
 struct State {
-  uint32_t prefix[3];  // key bits decided after pass 0, 1, 2 (right-aligned)
-  uint32_t k_rem[3];   // entries still to take from the bin picked in that pass
-  uint32_t overflow;   // a wave found more candidates than its list holds: the write launch re-reads
-  uint32_t pad[57];
+  uint32_t prefix[3];  // level-0 bin, level-1 digit, threshold key
+  uint32_t k_rem[3];   // entries still to take from the bin picked at that level
+  uint32_t overflow;   // a level-0 list overflowed (or no lists were asked for)
+  uint32_t overflow2;  // a list rebuilt by count overflowed: write re-reads the priorities
+  uint32_t hint_bin;   // candidates are the entries whose level-0 bin is >= this
+  uint32_t full;       // levels 1, 2, count stream the priorities instead of the lists
+  uint32_t lo0, hi0;   // smallest and largest key of the picked level-0 bin
+  BinMap map;
+  uint32_t pad[45];
 };
 static_assert(sizeof(State) == 256, "State is the 256-byte header of the workspace");
 
@@ -43,190 +100,176 @@ __device__ __forceinline__ uint32_t order_key(float f) {
   return key;
 }
 
-constexpr int kStep = kWave * 4;  // elements one wave handles per step (one float4 per lane)
-constexpr int kAhead = 4;         // steps whose loads are in flight together
-
-// Geometry of the compaction launches: `ranges` workgroups, every wave owns wave_len consecutive
-// elements (a multiple of kStep) and a candidate list of list_cap entries.
-struct Geom {
-  int64_t ranges, wave_len, list_cap;
-};
-
-Geom geom(int64_t n, int64_t k) {
-  Geom g;
-  g.ranges = ceil_div64(n > 0 ? n : 1, (int64_t)kWavesPerBlock * kAhead * kStep);
-  if (g.ranges > kMaxRanges) g.ranges = kMaxRanges;
-  g.wave_len = ceil_div64(ceil_div64(n > 0 ? n : 1, g.ranges * kWavesPerBlock), kStep) * kStep;
-  g.ranges = ceil_div64(n > 0 ? n : 1, g.wave_len * kWavesPerBlock);
-  // four times a wave's fair share of the k selected entries, at least 64, never more than the
-  // wave has elements; clustered maxima or many ties overflow it and take the re-reading path
-  const int64_t waves = g.ranges * kWavesPerBlock;
-  int64_t cap = ceil_div64(4 * ceil_div64(k > 0 ? k : 1, waves), 64) * 64;
-  if (cap < 64) cap = 64;
-  if (cap > g.wave_len) cap = g.wave_len;
-  g.list_cap = cap;
-  return g;
-}
-
 // the priority whose order_key is `key` (for +-0.0: +0.0)
 __device__ __forceinline__ float key_to_float(uint32_t key) {
   return __uint_as_float((key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
 }
 
+// Float bounds of a range of keys: float order = key order for non-NaN values.  The keys beyond
+// the infinities decode to NaN, with which every compare is false, and the key just below
+// +-0.0's does not exist (-0.0 ranks with +0.0), so the bounds stop short of them.
+constexpr uint32_t kKeyPosInf = 0xff800000u, kKeyNegInf = 0x007fffffu;
+__device__ __forceinline__ float lower_bound_float(uint32_t lo_key) {
+  if (lo_key < kKeyNegInf) lo_key = kKeyNegInf;
+  if (lo_key > kKeyPosInf) lo_key = kKeyPosInf;
+  return key_to_float(lo_key);
+}
+__device__ __forceinline__ float upper_bound_float(uint32_t hi_key) {
+  if (hi_key == 0x7fffffffu) hi_key = 0x7ffffffeu;
+  if (hi_key > kKeyPosInf) hi_key = kKeyPosInf;
+  if (hi_key < kKeyNegInf) hi_key = kKeyNegInf;
+  return key_to_float(hi_key);
+}
+
+constexpr int kStep = kWave * 4;  // elements one wave handles per step (one float4 per lane)
+constexpr int kAhead = 4;         // steps whose loads are in flight together
+
+// Every wave owns wave_len consecutive elements (a multiple of kStep) and a candidate list of
+// list_cap entries; `blocks` workgroups of 16 waves cover the input.
+struct Geom {
+  int64_t blocks, wave_len, list_cap;
+};
+
+Geom geom(int64_t n, int64_t k) {
+  Geom g;
+  const int64_t nn = n > 0 ? n : 1;
+  g.wave_len = ceil_div64(ceil_div64(nn, (int64_t)kMaxBlocks * kWavesPerBlock), kStep) * kStep;
+  g.blocks = ceil_div64(nn, g.wave_len * kWavesPerBlock);
+  // eight times a wave's fair share of k, between 256 and 1024 entries, never more than the wave
+  // has elements; clustered maxima or masses of ties overflow it and take the streaming path
+  const int64_t waves = g.blocks * kWavesPerBlock;
+  int64_t cap = ceil_div64(8 * ceil_div64(k > 0 ? k : 1, waves), 64) * 64;
+  if (cap < 256) cap = 256;
+  if (cap > 1024) cap = 1024;  // (level 0 itself lists at most kQueueCap = 512 per wave)
+  if (cap > g.wave_len) cap = g.wave_len;
+  g.list_cap = cap;
+  return g;
+}
+
 struct Layout {
-  size_t hist, desc, lists, ckey, cidx, skey, sidx, tkey, tidx, shist, total;
+  size_t hist0, hist1, hist2, wg_bins, boff, wave_listed, wave_ge, block_ge, lists, cidx,
+      cand, cand2, fin, cseg, ckey, skey, sidx, tkey, tidx, shist, zero_begin, zero_end, total;
 };
 
 Layout layout(int64_t n, int64_t k) {
   Layout l;
-  const size_t kk = align_up((size_t)(k > 0 ? k : 1) * 4, 256);
   const Geom g = geom(n, k);
+  const size_t kk = k > 0 ? (size_t)k : 1;
   size_t o = sizeof(State);
-  l.hist = o;  o += 3 * kHistBins * sizeof(uint32_t);
-  l.desc = o;  o += (size_t)kMaxRanges * (kWavesPerBlock + 1) * 8;  // wave and workgroup counts
-  l.lists = o; o += align_up((size_t)(g.ranges * kWavesPerBlock * g.list_cap) * 4, 256);
-  l.ckey = o;  o += kk;
-  l.cidx = o;  o += kk;
-  l.skey = o;  o += kk;
-  l.sidx = o;  o += kk;
-  l.tkey = o;  o += kk;
-  l.tidx = o;  o += kk;
-  l.shist = o; o += radix::hist_bytes(k);
+  l.zero_begin = o;
+  l.hist0 = o;  o += kBins0 * sizeof(uint32_t);
+  l.hist1 = o;  o += kBinsR * sizeof(uint32_t);
+  l.hist2 = o;  o += kBinsR * sizeof(uint32_t);
+  l.wg_bins = o; o += 2 * kMaxBlocks * sizeof(uint32_t);
+  l.zero_end = o;
+  l.boff = o;   o += kBins0 * sizeof(uint32_t);
+  l.wave_listed = o; o += (size_t)kMaxBlocks * kWavesPerBlock * sizeof(uint32_t);
+  l.wave_ge = o;     o += (size_t)kMaxBlocks * kWavesPerBlock * sizeof(uint64_t);
+  l.block_ge = o;    o += (size_t)kMaxBlocks * sizeof(uint64_t);
+  l.lists = o;  o += align_up((size_t)(g.blocks * kWavesPerBlock * g.list_cap) * 8, 256);
+  l.cidx = o;   o += align_up(kk * 4, 256);
+  l.cand = l.cand2 = l.fin = l.cseg = l.ckey = l.skey = l.sidx = l.tkey = l.tidx = l.shist = 0;
+  if (k <= kBucketMaxK) {
+    l.ckey = o;  o += align_up(kk * 4, 256);
+    l.cand = o;  o += align_up(kk * 8, 256);
+    l.cand2 = o; o += align_up(kk * 8, 256);
+    l.fin = o;   o += align_up(kk * 8, 256);
+    l.cseg = o;  o += align_up(kk, 256);
+  } else {
+    const size_t k4 = align_up(kk * 4, 256);
+    l.ckey = o; o += k4;
+    l.skey = o; o += k4;
+    l.sidx = o; o += k4;
+    l.tkey = o; o += k4;
+    l.tidx = o; o += k4;
+    l.shist = o; o += radix::hist_bytes(k);
+  }
   l.total = o;
   return l;
 }
 
-__global__ void zero_kernel(uint32_t *p, int64_t words) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < words) p[i] = 0u;
-}
-
-// Every thread of a 256-thread workgroup calls this: walk the histogram of pass PASS from the top
-// bin down and stop at the bin that holds the k_rem-th largest remaining key.  The result
-// (key prefix after this pass, entries still needed inside that bin) is returned to all threads.
-// The kernel that needs the result computes it itself instead of waiting for a launch of its own;
-// workgroup 0 also records it in `state` for the kernels after it.
+// Every thread of a kThreads workgroup calls this: walk a histogram of BINS bins from the top
+// bin down and stop at the bin that holds the k_rem-th largest remaining key.  Returns the bin
+// and the number of entries still needed inside it to all threads.  When boff is not null the
+// number of entries above every bin at or above the picked one is stored there (where the bin
+// starts in value order), and every non-empty one of those bins is entered into the segment
+// whose stretch of 2^seg_shift output places it starts in (wg_bins: highest bin + 1 and BINS -
+// lowest bin per segment, 0 = none).
+// With no such bin (only possible with NaN priorities, which the float compares of the later
+// levels do not count) the lowest bin is returned and nothing is taken off k_rem.
 struct Pick {
-  uint32_t prefix, k_rem;
+  uint32_t bin, k_rem;
 };
-template <int PASS, int THREADS = kBlock>
-__device__ __forceinline__ Pick pick_bin(int64_t k, State *state, const uint32_t *hist) {
-  constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
-  constexpr int kPerThread = kBinsHere / THREADS;
-  __shared__ uint32_t wsum[THREADS / kWave];
+template <int BINS>
+__device__ __forceinline__ Pick pick_bin(uint32_t k_rem, const uint32_t *hist, uint32_t *boff,
+                                         uint32_t *wg_bins = nullptr, int seg_shift = 0,
+                                         uint32_t rank2 = 0u, uint32_t *bin2 = nullptr) {
+  constexpr int kPerThread = BINS / kThreads > 0 ? BINS / kThreads : 1;
+  constexpr int kActive = BINS / kPerThread;  // threads that own bins
+  __shared__ uint32_t wsum[kWavesPerBlock];
   __shared__ Pick s_pick;
+  __shared__ uint32_t s_bin2;  // the bin that holds the rank2-th largest key (rank2 > 0)
+  __shared__ uint32_t s_seg[2 * kMaxBlocks];  // segment table, built in LDS and stored once
   const int tid = threadIdx.x;
-  const uint32_t prefix = PASS == 0 ? 0u : state->prefix[PASS == 0 ? 0 : PASS - 1];
-  const uint32_t k_rem = PASS == 0 ? (uint32_t)k : state->k_rem[PASS == 0 ? 0 : PASS - 1];
-  // thread t owns bins top-down: kBinsHere-1 - t*kPerThread - j
-  uint32_t c[kPerThread];
+  if (boff && tid < 2 * kMaxBlocks) s_seg[tid] = 0u;
+  uint32_t c[kPerThread];  // c[j] = count of bin BINS-1 - tid*kPerThread - j (top down)
   int tsum = 0;
+  if (kPerThread % 4 == 0) {
+    // the thread's bins are one contiguous run: 16-byte loads, reversed into top-down order
 #pragma unroll
-  for (int j = 0; j < kPerThread; ++j) {
-    c[j] = hist[kBinsHere - 1 - tid * kPerThread - j];
-    tsum += (int)c[j];
+    for (int v = 0; v < kPerThread / 4; ++v) {
+      const u32x4 q = *reinterpret_cast<const u32x4 *>(hist + BINS - (tid + 1) * kPerThread + v * 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) c[kPerThread - 1 - (v * 4 + e)] = q[e];
+    }
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) tsum += (int)c[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+      c[j] = tid < kActive ? hist[BINS - 1 - tid * kPerThread - j] : 0u;
+      tsum += (int)c[j];
+    }
   }
   const int inc = wave_inclusive_sum(tsum);
   if ((tid & 63) == 63) wsum[tid >> 6] = (uint32_t)inc;
-  // fallback when no bin holds the k_rem-th key (only possible with NaN priorities, which the
-  // float compares of the later passes do not count): the lowest bin, nothing taken off k_rem
   if (tid == 0) {
-    s_pick.prefix = PASS == 0 ? 0u : (PASS == 1 ? (prefix << 11) : (prefix << 10));
+    s_pick.bin = 0u;
     s_pick.k_rem = k_rem;
+    s_bin2 = 0u;
   }
   __syncthreads();
   uint32_t running = (uint32_t)(inc - tsum);
   for (int w = 0; w < (tid >> 6); ++w) running += wsum[w];
 #pragma unroll
   for (int j = 0; j < kPerThread; ++j) {
-    if (running < k_rem && running + c[j] >= k_rem) {
-      const uint32_t bin = (uint32_t)(kBinsHere - 1 - tid * kPerThread - j);
-      s_pick.prefix = PASS == 0 ? bin : (PASS == 1 ? ((prefix << 11) | bin) : ((prefix << 10) | bin));
-      s_pick.k_rem = k_rem - running;
+    const uint32_t bin = (uint32_t)(BINS - 1 - tid * kPerThread - j);
+    if (tid < kActive && running < k_rem) {
+      // a bin at or above the picked one: everything counted before it is selected
+      if (boff) {
+        boff[bin] = running;
+        if (c[j] != 0u) {  // the segment in whose stretch of the output the bin starts
+          const uint32_t w = running >> seg_shift;
+          atomicMax(&s_seg[2 * w], bin + 1u);
+          atomicMax(&s_seg[2 * w + 1], (uint32_t)BINS - bin);
+        }
+      }
+      if (running + c[j] >= k_rem) {
+        s_pick.bin = bin;
+        s_pick.k_rem = k_rem - running;
+      }
     }
+    if (rank2 != 0u && tid < kActive && running < rank2 && running + c[j] >= rank2) s_bin2 = bin;
     running += c[j];
   }
   __syncthreads();
+  if (boff && tid < 2 * kMaxBlocks) wg_bins[tid] = s_seg[tid];
+  if (bin2) *bin2 = s_bin2;
   const Pick r = s_pick;
-  if (blockIdx.x == 0 && tid == 0) {
-    state->prefix[PASS] = r.prefix;
-    state->k_rem[PASS] = r.k_rem;
-  }
+  __syncthreads();  // s_pick and wsum may be written again by a later call
   return r;
 }
 
-// PASS 0: bits 31..21, PASS 1: bits 20..10 of keys whose top 11 bits equal state->prefix,
-// PASS 2: bits 9..0 of keys whose top 22 bits equal state->prefix.  Workgroups count into LDS and
-// add their non-empty bins to the global histogram of this pass (hist; the previous pass's is
-// at hist - kHistBins); the bin of the previous pass is picked by every workgroup for itself.
-template <int PASS>
-__global__ __launch_bounds__(kHistThreads) void select_hist_kernel(const float *__restrict__ p,
-                                                             int64_t n, int64_t k, State *state,
-                                                             uint32_t *hist) {
-  constexpr int kBinsHere = PASS == 2 ? 1024 : 2048;
-  typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
-  __shared__ uint32_t h[kBinsHere];
-  const int tid = threadIdx.x;
-  for (int i = tid; i < kBinsHere; i += kHistThreads) h[i] = 0;
-  uint32_t prefix = 0u;
-  if (PASS == 1) prefix = pick_bin<0, kHistThreads>(k, state, hist - kHistBins).prefix;
-  if (PASS == 2) prefix = pick_bin<1, kHistThreads>(k, state, hist - kHistBins).prefix;
-  __syncthreads();
-
-  // Passes 1 and 2 count only the keys that start with `prefix`: about 1 % of the input.  Whether
-  // a priority is one of them is decided with two float compares against the bounds of that key
-  // range (float order = key order for non-NaN values, -0.0 == +0.0); the key itself is worked
-  // out only for the members.
-  constexpr int kLowBits = PASS == 1 ? 21 : 10;
-  uint32_t lo_key = PASS == 0 ? 0u : prefix << kLowBits;
-  uint32_t hi_key = PASS == 0 ? 0u : (lo_key | ((1u << kLowBits) - 1u));
-  if (hi_key == 0x7fffffffu) hi_key = 0x7ffffffeu;  // the key below +-0.0's: the zeros are not in this range
-  // the bins that hold +inf / -inf reach into keys that decode to NaN, with which every compare
-  // is false: the bounds stop at the keys of the infinities
-  constexpr uint32_t kKeyPosInf = 0xff800000u, kKeyNegInf = 0x007fffffu;
-  if (hi_key > kKeyPosInf) hi_key = kKeyPosInf;
-  if (lo_key < kKeyNegInf) lo_key = kKeyNegInf;
-  const float lo_f = key_to_float(lo_key), hi_f = key_to_float(hi_key);
-  auto count = [&](float f) {
-    if (PASS == 0) {
-      atomicAdd(&h[order_key(f) >> 21], 1u);
-    } else if (f >= lo_f && f <= hi_f) {
-      const uint32_t key = order_key(f);
-      atomicAdd(&h[PASS == 1 ? ((key >> 10) & 0x7ffu) : (key & 0x3ffu)], 1u);
-    }
-  };
-  const int64_t nvec = n >> 2;
-  constexpr int kLoads = 4;  // 16-byte loads in flight per thread
-  for (int64_t v0 = (int64_t)blockIdx.x * kHistThreads * kLoads + tid; v0 < nvec;
-       v0 += (int64_t)gridDim.x * kHistThreads * kLoads) {
-    f4 q[kLoads];
-#pragma unroll
-    for (int u = 0; u < kLoads; ++u) {
-      const int64_t v = v0 + (int64_t)u * kHistThreads;
-      q[u] = f4{0.0f, 0.0f, 0.0f, 0.0f};
-      if (v < nvec) q[u] = *reinterpret_cast<const f4 *>(p + (v << 2));
-    }
-#pragma unroll
-    for (int u = 0; u < kLoads; ++u) {
-      if (v0 + (int64_t)u * kHistThreads < nvec) {
-        count(q[u][0]);
-        count(q[u][1]);
-        count(q[u][2]);
-        count(q[u][3]);
-      }
-    }
-  }
-  if (blockIdx.x == 0 && tid < (int)(n & 3)) count(p[(nvec << 2) + tid]);
-  __syncthreads();
-  for (int i = tid; i < kBinsHere; i += kHistThreads)
-    if (h[i]) atomicAdd(&hist[i], h[i]);
-}
-
-// Ordered compaction in two launches with no waiting between workgroups.  The input is cut into
-// gridDim.x * 4 contiguous wave ranges of wave_len elements (a multiple of kStep).  The count
-// launch writes every wave's packed (greater << 31 | equal) count and every workgroup's total; the
-// write launch sums the totals of the workgroups before it, adds the counts of the waves before it
-// in its own workgroup, and walks its range again (now from L2 / MALL) placing the selected entries.
 typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
 
 __device__ __forceinline__ void load_quad(const float *__restrict__ p, int64_t e0, int64_t end,
@@ -240,27 +283,18 @@ __device__ __forceinline__ void load_quad(const float *__restrict__ p, int64_t e
   }
 }
 
-__global__ __launch_bounds__(kCompactThreads) void count_ranges_kernel(
-    const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist2,
-    int64_t wave_len, uint64_t *__restrict__ wave_counts, uint64_t *__restrict__ block_counts,
-    uint32_t *__restrict__ lists, int list_cap) {
-  __shared__ int64_t red[kWavesPerBlock];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
-  const int64_t begin = gw * wave_len;
-  const int64_t end = begin + wave_len < n ? begin + wave_len : n;
-  uint32_t *list = lists + gw * list_cap;
-  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  int listed = 0;         // candidates of this wave so far (wave-uniform)
-  bool overflow = false;  // wave-uniform
-  // the first loads are issued before the threshold is picked so that the two latencies overlap
+// A wave streams its range [begin, end): kAhead steps of one float4 per lane are in flight while
+// the previous kAhead are handed to f(e0, q) -- e0 the index of the lane's first element, q its
+// four values; elements at or beyond `end` hold 0 and must be skipped (e0 + j < end).  Every
+// lane of the wave calls f the same number of times, so f may ballot.
+template <typename F>
+__device__ __forceinline__ void stream_range(const float *__restrict__ p, int64_t begin,
+                                             int64_t end, int lane, F f) {
+  if (begin >= end) return;
   float q[kAhead][4];
 #pragma unroll
   for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
-  const float thr_f = key_to_float(pick_bin<2, kCompactThreads>(k, state, hist2).prefix);
-  uint32_t gt = 0, eq = 0;
   for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
-    // the next batch of loads is in flight while this one is classified and listed
     float qn[kAhead][4];
     const int64_t s1 = s0 + kAhead * kStep;
     if (s1 < end) {
@@ -270,166 +304,758 @@ __global__ __launch_bounds__(kCompactThreads) void count_ranges_kernel(
 #pragma unroll
     for (int a = 0; a < kAhead; ++a) {
       const int64_t e0 = s0 + (int64_t)a * kStep + lane * 4;
-      // every candidate (greater than, or equal to, the threshold) goes to the wave's list in
-      // index order as index | greater << 31; the write launch then never reads the priorities
-      bool sel[4];
-      uint32_t val[4];
-      int off[4], nc = 0;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // float compares order non-NaN priorities exactly like their keys (-0.0 == +0.0) at
-        // one instruction each
-        const bool above = q[a][j] > thr_f;
-        sel[j] = e0 + j < end && q[a][j] >= thr_f;
-        off[j] = nc;
-        nc += sel[j] ? 1 : 0;
-        gt += sel[j] && above;
-        eq += sel[j] && !above;
-        val[j] = (uint32_t)(e0 + j) | (above ? 0x80000000u : 0u);
-      }
-      if (wave_ballot(nc != 0) == 0ull) continue;
-      // candidates in the lanes before this one: nc <= 4 is three bits, one ballot per bit
-      // (independent instructions; a DPP scan is a chain of a dozen dependent ones)
-      const uint64_t b0 = wave_ballot((nc & 1) != 0), b1 = wave_ballot((nc & 2) != 0),
-                     b2 = wave_ballot((nc & 4) != 0);
-      const int before = __popcll(b0 & lt_mask) + 2 * __popcll(b1 & lt_mask) +
-                         4 * __popcll(b2 & lt_mask);
-      const int total = __popcll(b0) + 2 * __popcll(b1) + 4 * __popcll(b2);
-      if (listed + total > list_cap) {
-        overflow = true;
-      } else {
-        const int at = listed + before;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (sel[j]) list[at + off[j]] = val[j];
-      }
-      listed += total;
+      if (s0 + (int64_t)a * kStep < end) f(e0, q[a]);
     }
 #pragma unroll
     for (int a = 0; a < kAhead; ++a)
 #pragma unroll
       for (int j = 0; j < 4; ++j) q[a][j] = qn[a][j];
   }
-  if (overflow && lane == 0) state->overflow = 1u;  // same value from every overflowing wave
-  const int64_t w = wave_sum(((int64_t)gt << 31) | (int64_t)eq);
-  if (lane == 0) {
-    wave_counts[gw] = (uint64_t)w;
-    red[wave] = w;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    int64_t t = 0;
+}
+
+// Appends the lane's selected entries (sel[j], in element order) to the wave's list in index
+// order.  `listed` counts every candidate seen, also the ones that no longer fit (wave-uniform).
+__device__ __forceinline__ void list_append(uint64_t *list, int list_cap, int &listed,
+                                            bool &overflow, const bool sel[4],
+                                            const uint32_t key[4], int64_t e0, uint64_t lt_mask) {
+  int off[4], nc = 0;
 #pragma unroll
-    for (int i = 0; i < kWavesPerBlock; ++i) t += red[i];
-    block_counts[blockIdx.x] = (uint64_t)t;
+  for (int j = 0; j < 4; ++j) {
+    off[j] = nc;
+    nc += sel[j] ? 1 : 0;
+  }
+  if (wave_ballot(nc != 0) == 0ull) return;
+  // candidates in the lanes before this one: nc <= 4 is three bits, one ballot per bit
+  // (independent instructions; a DPP scan is a chain of a dozen dependent ones)
+  const uint64_t b0 = wave_ballot((nc & 1) != 0), b1 = wave_ballot((nc & 2) != 0),
+                 b2 = wave_ballot((nc & 4) != 0);
+  const int before = __popcll(b0 & lt_mask) + 2 * __popcll(b1 & lt_mask) + 4 * __popcll(b2 & lt_mask);
+  const int total = __popcll(b0) + 2 * __popcll(b1) + 4 * __popcll(b2);
+  if (listed + total > list_cap) {
+    overflow = true;
+  } else {
+    const int at = listed + before;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (sel[j]) list[at + off[j]] = ((uint64_t)key[j] << 32) | (uint32_t)(e0 + j);
+  }
+  listed += total;
+}
+
+// ---- prep: the sample, the bin map and the zeros ------------------------------------------------------
+// Workgroup 0 looks at kSamples priorities spread over the input (one per stride, at a hashed
+// offset inside it) and lays out the level-0 bins around them: the keys below the bin of the
+// `rank`-th largest sample (the hint; bins of the top 14 key bits) are binned coarsely, the
+// stretch from there to the largest sample as finely as kMidBins bins allow, the keys above with
+// what is left of the 16384 bins.  rank is set a few standard deviations beyond the sample's
+// share of k, so that the k-th largest priority of the whole input lies in the fine stretch
+// unless the sample misleads -- which costs time (the later levels stream the input again),
+// never correctness.  rank = 0: no sample, uniform bins; every entry is listed when list_all is
+// set (the lists are as long as the waves' ranges), none otherwise.  The other workgroups
+// clear the histograms.
+__global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict__ p, int64_t n,
+                                                        uint32_t rank, int list_all, int mid_bins,
+                                                        State *state, uint32_t *zero,
+                                                        int64_t zero_words) {
+  __shared__ __align__(16) uint32_t h[kBins0];
+  const int tid = threadIdx.x;
+  if (blockIdx.x > 0) {
+    const int64_t i = ((int64_t)(blockIdx.x - 1) * kThreads + tid) * 4;
+    if (i + 4 <= zero_words) {
+      *reinterpret_cast<u32x4 *>(zero + i) = u32x4{0u, 0u, 0u, 0u};
+    } else {
+      for (int64_t j = i; j < zero_words; ++j) zero[j] = 0u;
+    }
+    return;
+  }
+  constexpr int kPer = kSamples / kThreads;
+  float v[kPer];
+  if (rank != 0u) {
+    const int64_t stride = n / kSamples;  // >= 128 (the caller's condition for a sample), < 2^20
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const uint32_t s = (uint32_t)(tid + j * kThreads);
+      // a hashed offset inside the sample's stride: high half of hash * stride, no division
+      v[j] = p[(int64_t)s * stride + __umulhi(s * 2654435761u, (uint32_t)stride)];
+    }
+  }
+  if (tid < 3) state->prefix[tid] = 0u;
+  if (tid >= 3 && tid < 6) state->k_rem[tid - 3] = 0u;
+  if (tid == 6) state->overflow2 = 0u;
+  if (tid == 7) state->full = 0u;
+  if (tid == 8) state->overflow = (rank == 0u && !list_all) ? 1u : 0u;
+  BinMap map;
+  map.uniform = 1u;
+  map.a_end = map.b_last = map.nb0 = map.nc0 = map.b_shift = map.c_shift = 0u;
+  uint32_t hint = (rank == 0u && !list_all) ? kNoLists : 0u;
+  if (rank != 0u) {
+    for (int i = tid; i < kBins0; i += kThreads) h[i] = 0u;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) atomicAdd(&h[order_key(v[j]) >> kUniformShift], 1u);
+    __syncthreads();
+    uint32_t top14 = 0u;
+    const uint32_t hint14 = pick_bin<kBins0>(rank, h, nullptr, nullptr, 0, 1u, &top14).bin;
+    map.uniform = 0u;
+    map.a_end = (hint14 << kUniformShift) & ~((1u << kLowShift) - 1u);
+    map.b_last = ((top14 + 1u) << kUniformShift) - 1u;  // wraps to the last key for the top bin
+    const uint32_t span = map.b_last - map.a_end;
+    while ((span >> map.b_shift) >= (uint32_t)mid_bins) ++map.b_shift;
+    map.nb0 = map.a_end >> kLowShift;
+    map.nc0 = map.nb0 + (span >> map.b_shift) + 1u;
+    const uint32_t rest = 0xffffffffu - map.b_last;  // keys above the middle stretch
+    while (rest != 0u && map.nc0 + ((rest - 1u) >> map.c_shift) >= (uint32_t)kBins0) ++map.c_shift;
+    hint = map.nb0;  // the candidates: everything from the middle stretch upwards
+  }
+  if (tid == 0) {
+    state->hint_bin = hint;
+    state->map = map;
   }
 }
 
-template <bool DIRECT>
-__global__ __launch_bounds__(kCompactThreads) void write_ranges_kernel(
-    const float *__restrict__ p, int64_t n, int64_t k, const State *state, int64_t wave_len,
-    const uint64_t *__restrict__ wave_counts, const uint64_t *__restrict__ block_counts,
-    const uint32_t *__restrict__ lists, int list_cap, uint32_t *__restrict__ ckey,
-    uint32_t *__restrict__ cidx, float *__restrict__ values_out,
-    int64_t *__restrict__ indices_out) {
-  __shared__ int64_t red[kWavesPerBlock];
+// ---- level 0: ONE read of the priorities --------------------------------------------------------------
+// Every entry is counted in its level-0 bin (LDS histogram, flushed with atomics); the
+// candidates -- entries at or above the hint, about one in fifty -- are also listed per wave, in
+// index order, as key << 32 | index.  While streaming, a candidate is only dropped into the
+// wave's queue in LDS (value | index, in the order of arrival: nearly every wave step holds one
+// or two candidates, so whatever is done per candidate there is paid per step); after the
+// stream the wave orders its queue by index, bins the candidates and writes the list, all lanes
+// busy.  A candidate that finds the queue full is binned at once and the lists are given up.
+constexpr int kQueueCap = 512;  // candidates per wave held in LDS; longer lists overflow
+
+__global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restrict__ p, int64_t n,
+                                                          State *state,
+                                                          uint32_t *__restrict__ hist0,
+                                                          int64_t wave_len,
+                                                          uint32_t *__restrict__ wave_listed,
+                                                          uint64_t *__restrict__ lists, int list_cap) {
+  __shared__ __align__(16) uint32_t h[kBins0];
+  __shared__ uint64_t queue[kWavesPerBlock][kQueueCap];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < kBins0; i += kThreads) h[i] = 0u;
+  const uint32_t hint = state->hint_bin;
+  const BinMap map = state->map;
+  const bool want_lists = hint != kNoLists;
+  const float lo_f = lower_bound_float(
+      !want_lists ? kKeyPosInf : (map.uniform ? hint << kUniformShift : map.a_end));
+  // below the candidates every bin is key >> low_shift (the map's coarse stretch, or all bins
+  // of a uniform map)
+  const int low_shift = map.uniform ? kUniformShift : kLowShift;
+  const int cap = list_cap < kQueueCap ? list_cap : kQueueCap;
+  __syncthreads();
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   const int64_t begin = gw * wave_len;
   const int64_t end = begin + wave_len < n ? begin + wave_len : n;
-  const bool reread = state->overflow != 0u;  // some wave's list was too short: all waves re-read
-  float q[kAhead][4];
-  if (reread) {
+  uint64_t *list = lists + gw * list_cap;
+  uint64_t *wq = queue[wave];
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  uint32_t nq = 0;  // candidates of the wave so far (wave-uniform)
+  stream_range(p, begin, end, lane, [&](int64_t e0, const float q[4]) {
+    uint32_t rem = 0;  // bit j: element j of the lane is a candidate
 #pragma unroll
-    for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
+    for (int j = 0; j < 4; ++j) {
+      const bool valid = e0 + j < end;
+      const bool cand = want_lists && valid && q[j] >= lo_f;
+      rem |= cand ? 1u << j : 0u;
+      // everything else goes to its coarse bin right away
+      if (valid && !cand) atomicAdd(&h[order_key(q[j]) >> low_shift], 1u);
+    }
+    uint64_t with;  // lanes that still hold a candidate; a lane rarely has two: one round
+    while ((with = wave_ballot(rem != 0u)) != 0ull) {
+      if (rem != 0u) {
+        const int j = __ffs((int)rem) - 1;
+        rem &= rem - 1u;
+        const float x = j == 0 ? q[0] : (j == 1 ? q[1] : (j == 2 ? q[2] : q[3]));
+        const uint32_t at = nq + (uint32_t)__popcll(with & lt_mask);
+        if (at < (uint32_t)cap)
+          wq[at] = ((uint64_t)__float_as_uint(x) << 32) | (uint32_t)(e0 + j);
+        else
+          atomicAdd(&h[bin_of(map, order_key(x))], 1u);
+      }
+      nq += (uint32_t)__popcll(with);
+    }
+  });
+  if (want_lists) {
+    // the wave's queue: ordered by index (every entry counts the smaller ones), binned, listed
+    const uint32_t m_all = nq;
+    const uint32_t m = m_all < (uint32_t)cap ? m_all : (uint32_t)cap;
+    for (uint32_t i = lane; i < m; i += kWave) {
+      const uint64_t mine = wq[i];
+      const uint32_t index = (uint32_t)mine;
+      uint32_t r = 0;
+      const uint32_t m8 = m & ~7u;
+      for (uint32_t j = 0; j < m8; j += 8) {  // eight LDS reads in flight
+        uint32_t x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = (uint32_t)wq[j + u];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) r += x[u] < index;
+      }
+      for (uint32_t j = m8; j < m; ++j) r += (uint32_t)wq[j] < index;
+      const uint32_t key = order_key(__uint_as_float((uint32_t)(mine >> 32)));
+      atomicAdd(&h[bin_of(map, key)], 1u);
+      list[r] = ((uint64_t)key << 32) | index;
+    }
+    if (lane == 0) {
+      wave_listed[gw] = m;
+      if (m_all > (uint32_t)cap) state->overflow = 1u;  // same value from every overflowing wave
+    }
   }
-  const float thr_f = key_to_float(state->prefix[2]);
-  const uint32_t need_eq = state->k_rem[2];
-
-  int64_t part = 0;
-  for (int j = tid; j < (int)blockIdx.x; j += kCompactThreads) part += (int64_t)block_counts[j];
-  const int64_t pw = wave_sum(part);
-  if (lane == 0) red[wave] = pw;
   __syncthreads();
-  int64_t excl = 0;
+  for (int i = tid; i < kBins0; i += kThreads)
+    if (h[i]) atomicAdd(&hist0[i], h[i]);
+}
+
+// ---- levels 1 and 2: histograms inside the picked bin ------------------------------------------------
+// The keys of the picked level-0 bin are lo0 .. hi0; in `bits0` bits they can differ (at most 21).
+// LEVEL 1: picks the level-0 bin from hist0 (and decides whether the lists can be used: the hint
+// held when the picked bin is not below the hint bin); counts the top min(bits0, 11) of those
+// bits over the members of the bin.  LEVEL 2: picks the level-1 digit from hist1; counts the
+// remaining bits (at most 10) over the keys that share bin and digit.
+__device__ __forceinline__ int bits_of(uint32_t span) { return span ? 32 - __builtin_clz(span) : 0; }
+__device__ __forceinline__ int level1_shift(int bits0) { return bits0 > 11 ? bits0 - 11 : 0; }
+
+template <int LEVEL>
+__global__ __launch_bounds__(kThreads) void member_hist_kernel(
+    const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist_prev,
+    uint32_t *__restrict__ hist_out, uint32_t *boff, uint32_t *wg_bins, int seg_shift,
+    int64_t wave_len, const uint32_t *__restrict__ wave_listed,
+    const uint64_t *__restrict__ lists, int list_cap) {
+  __shared__ uint32_t h[kBinsR];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < kBinsR; i += kThreads) h[i] = 0u;
+  // the wave's list does not depend on the pick: its length and first stretch are asked for
+  // before the histogram is walked (used only when the lists are in use)
+  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const uint64_t *list = lists + gw * list_cap;
+  const int m_pre = (int)wave_listed[gw];
+  const uint64_t ent_pre = list[lane];
+  uint32_t lo, hi;  // the keys that are counted
+  int shift;        // digit = (key - lo) >> shift
+  bool full;
+  if (LEVEL == 1) {
+    const Pick r = pick_bin<kBins0>((uint32_t)k, hist_prev, blockIdx.x == 0 ? boff : nullptr,
+                                    wg_bins, seg_shift);
+    const BinMap map = state->map;
+    lo = bin_lo_key(map, r.bin);
+    hi = bin_hi_key(map, r.bin);
+    shift = level1_shift(bits_of(hi - lo));
+    full = state->overflow != 0u || r.bin < state->hint_bin;
+    if (blockIdx.x == 0 && tid == 0) {
+      state->prefix[0] = r.bin;
+      state->k_rem[0] = r.k_rem;
+      state->full = full ? 1u : 0u;
+      state->lo0 = lo;
+      state->hi0 = hi;
+    }
+  } else {
+    const Pick r = pick_bin<kBinsR>(state->k_rem[0], hist_prev, nullptr);
+    const uint32_t lo0 = state->lo0, hi0 = state->hi0;
+    const int shift1 = level1_shift(bits_of(hi0 - lo0));
+    lo = lo0 + (r.bin << shift1);
+    hi = lo + ((1u << shift1) - 1u);
+    if (hi > hi0 || hi < lo) hi = hi0;
+    shift = 0;
+    full = state->full != 0u;
+    if (blockIdx.x == 0 && tid == 0) {
+      state->prefix[1] = r.bin;
+      state->k_rem[1] = r.k_rem;
+    }
+  }
+  __syncthreads();
+  if (!full) {
+    const int m = m_pre;
+    for (int c0 = 0; c0 < m; c0 += kWave) {
+      if (c0 + lane < m) {
+        const uint32_t key = (uint32_t)((c0 == 0 ? ent_pre : list[c0 + lane]) >> 32);
+        if (key >= lo && key <= hi) atomicAdd(&h[(key - lo) >> shift], 1u);
+      }
+    }
+  } else {
+    // membership by two float compares against the bounds of the key range; the key itself is
+    // worked out only for the members
+    const float lo_f = lower_bound_float(lo);
+    const float hi_f = upper_bound_float(hi);
+    const int64_t begin = gw * wave_len;
+    const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+    stream_range(p, begin, end, lane, [&](int64_t e0, const float q[4]) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (e0 + j < end && q[j] >= lo_f && q[j] <= hi_f) {
+          const uint32_t key = order_key(q[j]);
+          if (key >= lo && key <= hi) atomicAdd(&h[(key - lo) >> shift], 1u);
+        }
+      }
+    });
+  }
+  __syncthreads();
+  for (int i = tid; i < kBinsR; i += kThreads)
+    if (h[i]) atomicAdd(&hist_out[i], h[i]);
+}
+
+// ---- count: threshold, then (greater, equal) per wave and workgroup ---------------------------------
+// Packed counts: greater << 32 | equal.  When the levels before streamed the priorities, this
+// launch does too and lists every wave's entries at or above the threshold on the way.
+__global__ __launch_bounds__(kThreads) void count_kernel(
+    const float *__restrict__ p, int64_t n, State *state, const uint32_t *hist2, int64_t wave_len,
+    uint32_t *__restrict__ wave_listed, uint64_t *__restrict__ lists, int list_cap,
+    uint64_t *__restrict__ wave_ge, uint64_t *__restrict__ block_ge) {
+  __shared__ uint64_t red[kWavesPerBlock];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  uint64_t *list = lists + gw * list_cap;
+  const int m_pre = (int)wave_listed[gw];  // asked for before the pick; used with the lists only
+  const uint64_t ent_pre = list[lane];
+  const Pick r = pick_bin<kBinsR>(state->k_rem[1], hist2, nullptr);
+  const uint32_t thr =
+      state->lo0 + (state->prefix[1] << level1_shift(bits_of(state->hi0 - state->lo0))) + r.bin;
+  if (blockIdx.x == 0 && tid == 0) {
+    state->prefix[2] = thr;
+    state->k_rem[2] = r.k_rem;
+  }
+  const bool full = state->full != 0u;
+  uint32_t gt = 0, eq = 0;
+  if (!full) {
+    const int m = m_pre;
+    for (int c0 = 0; c0 < m; c0 += kWave) {
+      if (c0 + lane < m) {
+        const uint32_t key = (uint32_t)((c0 == 0 ? ent_pre : list[c0 + lane]) >> 32);
+        gt += key > thr;
+        eq += key == thr;
+      }
+    }
+  } else {
+    const float thr_f = key_to_float(thr);
+    const int64_t begin = gw * wave_len;
+    const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    int listed = 0;
+    bool overflow = false;
+    stream_range(p, begin, end, lane, [&](int64_t e0, const float q[4]) {
+      bool sel[4];
+      uint32_t key[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // float compares order non-NaN priorities exactly like their keys (-0.0 == +0.0)
+        const bool above = q[j] > thr_f;
+        sel[j] = e0 + j < end && q[j] >= thr_f;
+        gt += sel[j] && above;
+        eq += sel[j] && !above;
+        key[j] = above ? order_key(q[j]) : thr;
+      }
+      list_append(list, list_cap, listed, overflow, sel, key, e0, lt_mask);
+    });
+    if (lane == 0) wave_listed[gw] = (uint32_t)listed;
+    if (overflow && lane == 0) state->overflow2 = 1u;
+  }
+  const int64_t w = wave_sum((int64_t)(((uint64_t)gt << 32) | (uint64_t)eq));
+  if (lane == 0) {
+    wave_ge[gw] = (uint64_t)w;
+    red[wave] = (uint64_t)w;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    uint64_t t = 0;
+#pragma unroll
+    for (int i = 0; i < kWavesPerBlock; ++i) t += red[i];
+    block_ge[blockIdx.x] = t;
+  }
+}
+
+// ---- write: ordered compaction -----------------------------------------------------------------------
+enum Flavour {
+  kDirect,  // indices_out / values_out in index order
+  kPairs,   // (inverted key, index) in index order for the LSD radix sort
+  kBucket   // (key, index) in index order for the bucket sort; ties at T go straight to the output's tail
+};
+
+template <int FLAVOUR>
+__global__ __launch_bounds__(kThreads) void write_kernel(
+    const float *__restrict__ p, int64_t n, int64_t k, const State *state, int64_t wave_len,
+    const uint32_t *__restrict__ wave_listed, const uint64_t *__restrict__ lists, int list_cap,
+    const uint64_t *__restrict__ wave_ge, const uint64_t *__restrict__ block_ge,
+    uint32_t *__restrict__ ckey, uint32_t *__restrict__ cidx, const uint32_t *__restrict__ boff,
+    int seg_shift, uint8_t *__restrict__ cseg, float *__restrict__ values_out,
+    int64_t *__restrict__ indices_out) {
+  __shared__ uint64_t red[kWavesPerBlock];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const uint64_t *list = lists + gw * list_cap;
+  const int m_pre = (int)wave_listed[gw];
+  const uint64_t ent_pre = list[lane];
+  const uint32_t thr = state->prefix[2];
+  const uint32_t need_eq = state->k_rem[2];
+  const bool reread = state->full != 0u && state->overflow2 != 0u;
+  const BinMap map = state->map;
+
+  // counts of the workgroups before this one (at most kMaxBlocks), then of the waves before
+  // this one in its own workgroup
+  uint64_t part = 0;
+  if (tid < (int)blockIdx.x) part = block_ge[tid];
+  const int64_t pw = wave_sum((int64_t)part);
+  if (lane == 0) red[wave] = (uint64_t)pw;
+  __syncthreads();
+  uint64_t excl = 0;
 #pragma unroll
   for (int i = 0; i < kWavesPerBlock; ++i) excl += red[i];
-  // plus the waves before this one in its own workgroup
-  int64_t own = 0;
-  if (lane < wave) own = (int64_t)wave_counts[(int64_t)blockIdx.x * kWavesPerBlock + lane];
-  excl += wave_sum(own);
-  uint32_t gt_run = (uint32_t)(excl >> 31), eq_run = (uint32_t)(excl & 0x7fffffff);
+  uint64_t own = 0;
+  if (lane < wave) own = wave_ge[(int64_t)blockIdx.x * kWavesPerBlock + lane];
+  excl += (uint64_t)wave_sum((int64_t)own);
+  uint32_t gt_run = (uint32_t)(excl >> 32), eq_run = (uint32_t)excl;
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  const uint32_t ties_at = (uint32_t)k - need_eq;  // where the ties at T start in value order
 
-  auto emit = [&](uint32_t pos, int64_t index, float value, uint32_t key) {
-    if (pos >= (uint32_t)k) return;  // counts that NaN priorities put out of step never leave the outputs
-    if (DIRECT) {
-      indices_out[pos] = index;
-      if (values_out) values_out[pos] = value;
+  // pos = the entry's place in index order among the selected, e = its rank among the entries
+  // equal to T.
+  auto emit = [&](bool selected, bool is_eq, uint32_t pos, uint32_t e, uint32_t index, uint32_t key) {
+    selected = selected && pos < (uint32_t)k;  // out of step only with NaN priorities
+    if (FLAVOUR == kDirect) {
+      if (selected) {
+        indices_out[pos] = (int64_t)index;
+        if (values_out) values_out[pos] = p[index];
+      }
+    } else if (FLAVOUR == kPairs) {
+      if (selected) {
+        ckey[pos] = ~key;
+        cidx[pos] = index;
+      }
     } else {
-      ckey[pos] = ~key;
-      cidx[pos] = (uint32_t)index;
+      // ties at T are the smallest selected keys: they close the output, in index order; the
+      // bucket sort skips them (it takes keys above T only)
+      if (selected && is_eq && ties_at + e < (uint32_t)k) {
+        indices_out[ties_at + e] = (int64_t)index;
+        if (values_out) values_out[ties_at + e] = p[index];
+      }
+      if (selected) {
+        ckey[pos] = key;
+        cidx[pos] = index;
+        // the segment of the sort that takes the entry: the one in whose stretch of the
+        // output the entry's level-0 bin starts (ties at T belong to none)
+        cseg[pos] = is_eq ? (uint8_t)kNoSegment : (uint8_t)(boff[bin_of(map, key)] >> seg_shift);
+      }
     }
   };
 
   if (!reread) {
-    // the wave's candidates, in index order, from its list
-    const uint64_t mine = wave_counts[gw];
-    const int m = (int)(mine >> 31) + (int)(mine & 0x7fffffff);
-    const uint32_t *list = lists + gw * list_cap;
-    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    const int m = m_pre;
     for (int c0 = 0; c0 < m; c0 += kWave) {
       const bool valid = c0 + lane < m;
-      const uint32_t ent = valid ? list[c0 + lane] : 0u;
-      const bool is_gt = valid && (ent >> 31) != 0u, is_eq = valid && (ent >> 31) == 0u;
+      const uint64_t ent = valid ? (c0 == 0 ? ent_pre : list[c0 + lane]) : 0ull;
+      const uint32_t key = (uint32_t)(ent >> 32);
+      const bool is_gt = valid && key > thr, is_eq = valid && key == thr;
       const uint64_t bg = wave_ballot(is_gt), be = wave_ballot(is_eq);
       const uint32_t g = gt_run + (uint32_t)__popcll(bg & lt_mask);
       const uint32_t e = eq_run + (uint32_t)__popcll(be & lt_mask);
-      if (is_gt || (is_eq && e < need_eq)) {
-        const uint32_t index = ent & 0x7fffffffu;
-        const float value = p[index];
-        emit(g + (e < need_eq ? e : need_eq), (int64_t)index, value, order_key(value));
-      }
+      const bool selected = is_gt || (is_eq && e < need_eq);
+      emit(selected, is_eq, g + (e < need_eq ? e : need_eq), e, (uint32_t)ent, key);
       gt_run += (uint32_t)__popcll(bg);
       eq_run += (uint32_t)__popcll(be);
     }
     return;
   }
 
-  for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
-    if (s0 != begin) {
+  const float thr_f = key_to_float(thr);
+  const int64_t begin = gw * wave_len;
+  const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+  stream_range(p, begin, end, lane, [&](int64_t e0, const float q[4]) {
+    int s = 0;  // packed counts of the lane's four entries: greater << 16 | equal
 #pragma unroll
-      for (int a = 0; a < kAhead; ++a) load_quad(p, s0 + (int64_t)a * kStep + lane * 4, end, q[a]);
+    for (int j = 0; j < 4; ++j)
+      if (e0 + j < end) s += q[j] > thr_f ? (1 << 16) : (q[j] == thr_f ? 1 : 0);
+    if (wave_ballot(s != 0) == 0ull) return;
+    const int inc = wave_inclusive_sum(s);
+    const int total = wave_read_lane(inc, kWave - 1);
+    const int before = inc - s;
+    uint32_t g = gt_run + ((uint32_t)before >> 16);
+    uint32_t e = eq_run + ((uint32_t)before & 0xffffu);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool valid = e0 + j < end;
+      const bool is_gt = valid && q[j] > thr_f, is_eq = valid && q[j] == thr_f;
+      const bool selected = is_gt || (is_eq && e < need_eq);
+      emit(selected, is_eq, g + (e < need_eq ? e : need_eq), e, (uint32_t)(e0 + j),
+           is_gt ? order_key(q[j]) : thr);
+      g += is_gt;
+      e += is_eq;
     }
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a) {
-      const int64_t e0 = s0 + (int64_t)a * kStep + lane * 4;
-      int s = 0;  // packed counts of the lane's four entries: greater << 16 | equal
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (e0 + j < end) s += q[a][j] > thr_f ? (1 << 16) : (q[a][j] == thr_f ? 1 : 0);
-      if (wave_ballot(s != 0) == 0ull) continue;
-      const int inc = wave_inclusive_sum(s);
-      const int total = wave_read_lane(inc, kWave - 1);
-      const int before = inc - s;
-      uint32_t g = gt_run + ((uint32_t)before >> 16);
-      uint32_t e = eq_run + ((uint32_t)before & 0xffffu);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (e0 + j < end) {
-          const bool is_gt = q[a][j] > thr_f, is_eq = q[a][j] == thr_f;
-          if (is_gt || (is_eq && e < need_eq))
-            emit(g + (e < need_eq ? e : need_eq), e0 + j, q[a][j], order_key(q[a][j]));
-          g += is_gt;
-          e += is_eq;
+    gt_run += (uint32_t)total >> 16;
+    eq_run += (uint32_t)total & 0xffffu;
+  });
+}
+
+// ---- value order: segments gathered and sorted --------------------------------------------------------
+// The selected entries arrive in index order as (key, index).  The level-0 histogram says where
+// every level-0 bin starts in the value-ordered output; bins whose start falls into the same
+// stretch of 2^seg_shift output places form the segment of one workgroup (a run of neighbouring
+// bins: workgroup w owns the bins wg_bins[w]).  The workgroup reads all k keys once, keeps the
+// entries above T inside its key range -- in LDS when they fit, else in its stretch of a
+// global buffer; the places come from a cursor of its own in LDS (global atomics that meet on an
+// address are served one after the other by the memory side) --, sorts them, and writes its
+// stretch of the output.  An entry is key << 32 | ~index, so a larger entry comes earlier in
+// value order (ties: smaller index first) and no two are equal.  The sort is a most-significant-
+// digit radix sort from the highest bit in which the segment's keys can differ: counting sort on
+// 9 bits, groups of up to kSmallGroup entries are ranked directly (every entry counts the larger
+// ones), larger groups (equal or nearly equal keys) go down another 9 bits from a stack.
+constexpr int kLdsEntries = 8192;  // entries per LDS buffer of the segment sort
+constexpr int kStack = 1024;
+
+constexpr int kSortBins = 512;  // 9-bit digits
+struct SortShared {
+  uint32_t cnt[kSortBins + 1];
+  uint32_t start[kSortBins + 1];
+  uint32_t wsum[kSortThreads / kWave];
+  uint32_t stk_off[kStack], stk_len[kStack];
+  uint8_t stk_bits[kStack];   // low bits of the entries still undecided inside the group
+  uint8_t stk_flip[kStack];   // the group sits in the second buffer
+  int stk_top;
+};
+
+// number of entries of src[lo, hi) larger than `mine`
+__device__ __forceinline__ uint32_t larger_in(const uint64_t *src, uint32_t lo, uint32_t hi,
+                                              uint64_t mine) {
+  uint32_t r = 0;
+  uint32_t j = lo;
+  for (; j + 4 <= hi; j += 4) {
+    const uint64_t x0 = src[j], x1 = src[j + 1], x2 = src[j + 2], x3 = src[j + 3];
+    r += (x0 > mine) + (x1 > mine) + (x2 > mine) + (x3 > mine);
+  }
+  for (; j < hi; ++j) r += src[j] > mine;
+  return r;
+}
+
+// Sorts the m entries a[0, m) (descending; only their low `bits` bits can differ) with b as the
+// second buffer and stores them to fin[0, m); called by every thread of the workgroup.  The two
+// callers pass either the LDS buffers or global ones, so that after inlining every access has a
+// known address space.
+__device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t m, int bits,
+                                             uint64_t *__restrict__ fin, SortShared &sh) {
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    sh.stk_off[0] = 0u;
+    sh.stk_len[0] = m;
+    sh.stk_bits[0] = (uint8_t)bits;
+    sh.stk_flip[0] = 0;
+    sh.stk_top = 1;
+  }
+  __syncthreads();
+  while (true) {
+    const int top = sh.stk_top;
+    if (top == 0) break;
+    const uint32_t off = sh.stk_off[top - 1], len = sh.stk_len[top - 1];
+    const int rem = sh.stk_bits[top - 1];
+    const bool flip = sh.stk_flip[top - 1] != 0;
+    __syncthreads();
+    if (tid == 0) sh.stk_top = top - 1;
+    const uint64_t *src = flip ? b : a;
+    uint64_t *dst = flip ? a : b;
+    if (len <= (uint32_t)kSmallGroup || rem == 0) {
+      for (uint32_t i = tid; i < len; i += kSortThreads) {
+        const uint64_t mine = src[off + i];
+        fin[off + larger_in(src, off, off + len, mine)] = mine;
+      }
+      __syncthreads();
+      continue;
+    }
+    const int nb = rem < 9 ? rem : 9;
+    const int shift = rem - nb;
+    const uint32_t mask = (1u << nb) - 1u;
+    // counting sort of src[off, off+len) by the digit, largest digit first
+    for (int i = tid; i <= kSortBins; i += kSortThreads) sh.cnt[i] = 0u;
+    __syncthreads();
+#pragma unroll 4
+    for (uint32_t i = tid; i < len; i += kSortThreads)
+      atomicAdd(&sh.cnt[mask - (uint32_t)((src[off + i] >> shift) & mask)], 1u);
+    __syncthreads();
+    {
+      const uint32_t c = tid < kSortBins ? sh.cnt[tid] : 0u;  // the first kSortBins threads own a digit each
+      const int inc = wave_inclusive_sum((int)c);
+      if ((tid & 63) == 63) sh.wsum[tid >> 6] = (uint32_t)inc;
+      __syncthreads();
+      uint32_t before = (uint32_t)inc - c;
+      for (int w = 0; w < (tid >> 6); ++w) before += sh.wsum[w];
+      if (tid < kSortBins) {
+        sh.start[tid] = before;
+        sh.cnt[tid] = before;  // cursors
+      }
+      if (tid == kSortBins - 1) sh.start[kSortBins] = before + c;
+      __syncthreads();
+    }
+#pragma unroll 4
+    for (uint32_t i = tid; i < len; i += kSortThreads) {
+      const uint64_t ent = src[off + i];
+      const uint32_t d = mask - (uint32_t)((ent >> shift) & mask);
+      dst[off + atomicAdd(&sh.cnt[d], 1u)] = ent;
+    }
+    __syncthreads();
+    // groups: small ones are ranked and stored, large ones go down a level
+    for (uint32_t i = tid; i < len; i += kSortThreads) {
+      const uint64_t mine = dst[off + i];
+      const uint32_t d = mask - (uint32_t)((mine >> shift) & mask);
+      const uint32_t gs = sh.start[d], ge = sh.start[d + 1];
+      if (ge - gs <= (uint32_t)kSmallGroup || shift == 0) {
+        fin[off + gs + larger_in(dst, off + gs, off + ge, mine)] = mine;
+      } else if (i == gs) {
+        const int at = atomicAdd(&sh.stk_top, 1);
+        if (at < kStack) {
+          sh.stk_off[at] = off + gs;
+          sh.stk_len[at] = ge - gs;
+          sh.stk_bits[at] = (uint8_t)shift;
+          sh.stk_flip[at] = flip ? 0 : 1;
         }
       }
-      gt_run += (uint32_t)total >> 16;
-      eq_run += (uint32_t)total & 0xffffu;
     }
+    __syncthreads();
   }
 }
 
-// Final store of the value-ordered form, fused into the last digit of the candidate sort.
+__global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
+    const float *__restrict__ p, int64_t n, int64_t k, const State *state,
+    const uint32_t *__restrict__ hist0, const uint32_t *__restrict__ boff,
+    const uint32_t *__restrict__ wg_bins, const uint32_t *__restrict__ ckey,
+    const uint32_t *__restrict__ cidx, const uint8_t *__restrict__ cseg, uint64_t *buf0,
+    uint64_t *buf1, uint64_t *fin,
+    float *__restrict__ values_out, int64_t *__restrict__ indices_out) {
+  __shared__ uint64_t lds_a[kLdsEntries], lds_b[kLdsEntries];
+  __shared__ uint32_t s_cur;
+  __shared__ SortShared sh;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // The segment ids of the selected entries (a byte each; every workgroup reads them all) do
+  // not depend on what this workgroup owns: their loads go out first, sixteen ids per load.
+  const uint32_t kk = (uint32_t)k;
+  const uint32_t pattern = blockIdx.x * 0x01010101u;
+  constexpr int kLoads = 8;
+  u32x4 q[kLoads];
+#pragma unroll
+  for (int u = 0; u < kLoads; ++u) {
+    const uint32_t i0 = ((uint32_t)u * kSortThreads + tid) * 16;
+    q[u] = u32x4{~pattern, ~pattern, ~pattern, ~pattern};  // no byte matches
+    if (i0 + 16 <= kk) q[u] = *reinterpret_cast<const u32x4 *>(cseg + i0);
+  }
+  // this workgroup's bins (stored as highest bin + 1 and kBins0 - lowest bin; 0 = none)
+  const uint32_t hi1 = wg_bins[2 * blockIdx.x], loinv = wg_bins[2 * blockIdx.x + 1];
+  if (hi1 == 0u || loinv == 0u) return;
+  const uint32_t hi_bin = hi1 - 1u, lo_bin = (uint32_t)kBins0 - loinv;
+  const uint32_t b0 = state->prefix[0];
+  const uint32_t lo_count = lo_bin == b0 ? state->k_rem[0] - state->k_rem[2] : hist0[lo_bin];
+  const uint32_t out_lo = boff[hi_bin];
+  uint32_t out_hi = boff[lo_bin] + lo_count;
+  if (out_hi > kk) out_hi = kk;  // only out of step with NaN priorities
+  if (out_lo >= out_hi) return;
+  const uint32_t m = out_hi - out_lo;
+  // keys of the segment lie inside the bins' key range
+  const BinMap map = state->map;
+  const uint32_t lo_key = bin_lo_key(map, lo_bin);
+  const uint32_t hi_key = bin_hi_key(map, hi_bin);
+  const bool in_lds = m <= (uint32_t)kLdsEntries;
+  // the positions of the segment's entries are collected first: in LDS (the second buffer,
+  // two per word) or, for a segment that does not fit, in the second global buffer
+  uint32_t *pos_lds = reinterpret_cast<uint32_t *>(lds_b);
+  uint32_t *pos_glb = reinterpret_cast<uint32_t *>(buf1 + out_lo);
+  if (tid == 0) s_cur = 0u;
+  __syncthreads();
+
+  // one pass over the segment ids: words without this segment's id are dismissed four ids at a
+  // time; the first kLoads loads per thread are already under way
+  {
+    for (uint32_t r0 = 0; r0 < kk; r0 += kSortThreads * 16 * kLoads) {
+      if (r0 != 0u) {
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+          const uint32_t i0 = r0 + ((uint32_t)u * kSortThreads + tid) * 16;
+          q[u] = u32x4{~pattern, ~pattern, ~pattern, ~pattern};
+          if (i0 + 16 <= kk) q[u] = *reinterpret_cast<const u32x4 *>(cseg + i0);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kLoads; ++u) {
+        const uint32_t i0 = r0 + ((uint32_t)u * kSortThreads + tid) * 16;
+        if (i0 < kk && i0 + 16 > kk) {  // the ragged end of the ids: at most one thread
+          for (int e = 0; e < 16; ++e)
+            if (i0 + e < kk)
+              q[u][e >> 2] = (q[u][e >> 2] & ~(0xffu << (8 * (e & 3)))) |
+                             ((uint32_t)cseg[i0 + e] << (8 * (e & 3)));
+        }
+        uint32_t hits = 0;  // bit e: id e of the lane's sixteen is this segment's
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t t = q[u][w] ^ pattern;
+          if (((t - 0x01010101u) & ~t & 0x80808080u) != 0u) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (((t >> (8 * e)) & 0xffu) == 0u) hits |= 1u << (4 * w + e);
+          }
+        }
+        if (wave_ballot(hits != 0u) == 0ull) continue;
+        const int nc = __popc(hits);
+        const int inc = wave_inclusive_sum(nc);
+        uint32_t base = 0;
+        if (lane == kWave - 1) base = atomicAdd(&s_cur, (uint32_t)inc);
+        base = (uint32_t)__builtin_amdgcn_readlane((int)base, kWave - 1) + (uint32_t)(inc - nc);
+        while (hits) {
+          const int e = __ffs((int)hits) - 1;
+          hits &= hits - 1u;
+          if (base < m) {
+            if (in_lds) pos_lds[base] = i0 + (uint32_t)e; else pos_glb[base] = i0 + (uint32_t)e;
+          }
+          ++base;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // positions -> entries (key, inverted index), many gathers in flight
+  {
+    constexpr int kGathers = 8;
+    for (uint32_t i = tid; i < m; i += kSortThreads * kGathers) {
+      uint32_t pos[kGathers], key[kGathers], idx[kGathers];
+#pragma unroll
+      for (int u = 0; u < kGathers; ++u) {
+        const uint32_t iu = i + (uint32_t)u * kSortThreads;
+        pos[u] = iu < m ? (in_lds ? pos_lds[iu] : pos_glb[iu]) : kk;
+      }
+#pragma unroll
+      for (int u = 0; u < kGathers; ++u) {
+        key[u] = pos[u] < kk ? ckey[pos[u]] : 0u;
+        idx[u] = pos[u] < kk ? cidx[pos[u]] : 0u;
+      }
+#pragma unroll
+      for (int u = 0; u < kGathers; ++u) {
+        const uint32_t iu = i + (uint32_t)u * kSortThreads;
+        if (iu < m) {
+          const uint64_t ent = ((uint64_t)key[u] << 32) | (uint32_t)~idx[u];
+          if (in_lds) lds_a[iu] = ent; else buf0[out_lo + iu] = ent;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // bits of the entries that can differ inside the segment: the index, and the key below the
+  // highest bit in which the segment's smallest and largest key differ
+  const uint32_t diff = lo_key ^ hi_key;
+  const int bits = 32 + (diff ? 32 - __builtin_clz(diff) : 0);
+  if (in_lds)
+    sort_segment(lds_a, lds_b, m, bits, fin + out_lo, sh);
+  else
+    sort_segment(buf0 + out_lo, buf1 + out_lo, m, bits, fin + out_lo, sh);
+  __syncthreads();
+
+  // The segment's stretch of the output, in order.  The value follows from the key (the map is
+  // one to one) except for the two zeros, which share a key: those are read from the input.  (A
+  // gather of every value would be bound by the misses one CU can have in flight.)
+  for (uint32_t i = tid; i < m; i += kSortThreads) {
+    const uint64_t ent = fin[out_lo + i];
+    const uint32_t index = ~(uint32_t)ent, key = (uint32_t)(ent >> 32);
+    indices_out[out_lo + i] = (int64_t)index;
+    if (values_out)
+      values_out[out_lo + i] =
+          key != 0x80000000u ? key_to_float(key) : ((int64_t)index < n ? p[index] : 0.0f);
+  }
+}
+static_assert(kSortThreads >= kSortBins, "a thread per digit in the segment sort's scan");
+
+// Final store of the value-ordered form for k > kBucketMaxK, fused into the last digit of the
+// candidate sort.
 struct EmitSorted {
   static constexpr bool kActive = true;
   const float *p;
@@ -443,17 +1069,6 @@ struct EmitSorted {
     if (values) values[pos] = index < n ? p[index] : 0.0f;
   }
 };
-
-__global__ __launch_bounds__(kBlock) void emit_kernel(const float *__restrict__ p,
-                                                      const uint32_t *__restrict__ sidx, int64_t k,
-                                                      int64_t n, float *__restrict__ values_out,
-                                                      int64_t *__restrict__ indices_out) {
-  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (j >= k) return;
-  const uint32_t i = sidx[j];
-  indices_out[j] = (int64_t)i;
-  if (values_out) values_out[j] = (int64_t)i < n ? p[i] : 0.0f;
-}
 
 }  // namespace
 }  // namespace gearhip
@@ -475,60 +1090,89 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
     return GEAR_HIP_EWORKSPACE;
   char *ws = static_cast<char *>(workspace);
   State *state = reinterpret_cast<State *>(ws);
-  uint32_t *hist = reinterpret_cast<uint32_t *>(ws + l.hist);
-  hipStream_t st = as_stream(stream);
-
-  const int64_t zero_words = (int64_t)(l.desc / 4);  // header + histograms
-  zero_kernel<<<dim3((unsigned)ceil_div64(zero_words, 256)), dim3(256), 0, st>>>(
-      reinterpret_cast<uint32_t *>(ws), zero_words);
-  int64_t hblocks = ceil_div64(n, (int64_t)kHistThreads * 4 * 4);
-  if (hblocks < 1) hblocks = 1;
-  if (hblocks > kMaxHistBlocks) hblocks = kMaxHistBlocks;
-  const dim3 hgrid((unsigned)hblocks), hblock(kHistThreads), block(kBlock);
-  select_hist_kernel<0><<<hgrid, hblock, 0, st>>>(priorities, n, k, state, hist);
-  select_hist_kernel<1><<<hgrid, hblock, 0, st>>>(priorities, n, k, state, hist + kHistBins);
-  select_hist_kernel<2><<<hgrid, hblock, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins);
-  GEARHIP_RETURN_IF_LAUNCH_FAILED();
-
-  uint32_t *ckey = reinterpret_cast<uint32_t *>(ws + l.ckey);
+  uint32_t *hist0 = reinterpret_cast<uint32_t *>(ws + l.hist0);
+  uint32_t *hist1 = reinterpret_cast<uint32_t *>(ws + l.hist1);
+  uint32_t *hist2 = reinterpret_cast<uint32_t *>(ws + l.hist2);
+  uint32_t *boff = reinterpret_cast<uint32_t *>(ws + l.boff);
+  uint32_t *wave_listed = reinterpret_cast<uint32_t *>(ws + l.wave_listed);
+  uint64_t *wave_ge = reinterpret_cast<uint64_t *>(ws + l.wave_ge);
+  uint64_t *block_ge = reinterpret_cast<uint64_t *>(ws + l.block_ge);
+  uint64_t *lists = reinterpret_cast<uint64_t *>(ws + l.lists);
   uint32_t *cidx = reinterpret_cast<uint32_t *>(ws + l.cidx);
-  const bool direct = !sorted_by_value;
+  hipStream_t st = as_stream(stream);
   const Geom g = geom(n, k);
-  const int64_t ranges = g.ranges, wave_len = g.wave_len;
-  uint32_t *lists = reinterpret_cast<uint32_t *>(ws + l.lists);
-  uint64_t *wave_counts = reinterpret_cast<uint64_t *>(ws + l.desc);
-  uint64_t *block_counts = wave_counts + (size_t)kMaxRanges * kWavesPerBlock;
-  const dim3 cgrid((unsigned)ranges), cblock(kCompactThreads);
-  count_ranges_kernel<<<cgrid, cblock, 0, st>>>(priorities, n, k, state, hist + 2 * kHistBins,
-                                               wave_len, wave_counts, block_counts, lists,
-                                               (int)g.list_cap);
-  if (direct)
-    write_ranges_kernel<true><<<cgrid, cblock, 0, st>>>(priorities, n, k, state, wave_len, wave_counts,
-                                                       block_counts, lists, (int)g.list_cap, ckey,
-                                                       cidx, values_out, indices_out);
-  else
-    write_ranges_kernel<false><<<cgrid, cblock, 0, st>>>(priorities, n, k, state, wave_len,
-                                                        wave_counts, block_counts, lists,
-                                                        (int)g.list_cap, ckey, cidx, values_out,
-                                                        indices_out);
+
+  // The hint: rank of the sample that safely lies below the k-th largest priority -- the sample's
+  // expected share of k plus six standard deviations and a little.  No sample when the lists hold
+  // whole ranges anyway, when the input is small, or when k is a large part of it (the lists
+  // would hold most of the input: the levels stream instead).
+  const int list_all = g.list_cap >= g.wave_len ? 1 : 0;
+  uint32_t rank = 0;
+  if (!list_all && n >= 128 * (int64_t)kSamples && k <= n / 16 &&
+      env_int("GEAR_HIP_TOPK_HINT", 1) != 0) {
+    const double mu = (double)kSamples * (double)k / (double)n;
+    const double r = mu + 6.0 * __builtin_sqrt(mu) + 8.0;
+    if (r < kSamples / 4) rank = (uint32_t)r + 1u;
+  }
+  const int64_t zero_words = (int64_t)((l.zero_end - l.zero_begin) / 4);
+  const unsigned zero_blocks = (unsigned)ceil_div64(zero_words, (int64_t)kThreads * 4);
+  const dim3 block(kThreads), grid((unsigned)g.blocks);
+  // Fine bins pay off in the value-order sort (small, even segments) but cost level 0 an atomic
+  // per candidate when its histogram is flushed; the index-ordered selection takes coarse ones.
+  const int mid_bins = (sorted_by_value && k <= kBucketMaxK) ? kMidBins : kMidBinsCoarse;
+  prep_kernel<<<dim3(1 + zero_blocks), block, 0, st>>>(
+      priorities, n, rank, list_all, mid_bins, state,
+      reinterpret_cast<uint32_t *>(ws + l.zero_begin), zero_words);
+  level0_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len, wave_listed,
+                                        lists, (int)g.list_cap);
+  // value order by segments: workgroup w of the sort owns the bins that start in the output
+  // places [w << seg_shift, (w + 1) << seg_shift)
+  const bool by_segments = sorted_by_value && k <= kBucketMaxK;
+  int seg_shift = 0;
+  while ((k >> seg_shift) >= kNoSegment) ++seg_shift;  // segment ids stay below kNoSegment
+  uint32_t *wg_bins = reinterpret_cast<uint32_t *>(ws + l.wg_bins);
+  member_hist_kernel<1><<<grid, block, 0, st>>>(priorities, n, k, state, hist0, hist1,
+                                                by_segments ? boff : nullptr, wg_bins, seg_shift,
+                                                g.wave_len, wave_listed, lists, (int)g.list_cap);
+  member_hist_kernel<2><<<grid, block, 0, st>>>(priorities, n, k, state, hist1, hist2, nullptr,
+                                                nullptr, 0, g.wave_len, wave_listed, lists,
+                                                (int)g.list_cap);
+  count_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist2, g.wave_len, wave_listed, lists,
+                                       (int)g.list_cap, wave_ge, block_ge);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  if (direct) return 0;
+  uint8_t *cseg = reinterpret_cast<uint8_t *>(ws + l.cseg);
+#define GEARHIP_WRITE(F, CKEY)                                                                     \
+  write_kernel<F><<<grid, block, 0, st>>>(priorities, n, k, state, g.wave_len, wave_listed, lists,  \
+                                          (int)g.list_cap, wave_ge, block_ge, CKEY, cidx, boff,     \
+                                          seg_shift, cseg, values_out, indices_out)
+  if (!sorted_by_value) {
+    GEARHIP_WRITE(kDirect, nullptr);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  if (k <= kBucketMaxK) {
+    uint64_t *cand = reinterpret_cast<uint64_t *>(ws + l.cand);
+    uint64_t *cand2 = reinterpret_cast<uint64_t *>(ws + l.cand2);
+    uint32_t *bkey = reinterpret_cast<uint32_t *>(ws + l.ckey);
+    GEARHIP_WRITE(kBucket, bkey);
+    uint64_t *fin = reinterpret_cast<uint64_t *>(ws + l.fin);
+    segment_sort_kernel<<<dim3(kMaxBlocks), dim3(kSortThreads), 0, st>>>(
+        priorities, n, k, state, hist0, boff, wg_bins, bkey, cidx, cseg, cand, cand2, fin,
+        values_out, indices_out);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  uint32_t *ckey = reinterpret_cast<uint32_t *>(ws + l.ckey);
+  GEARHIP_WRITE(kPairs, ckey);
+#undef GEARHIP_WRITE
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
   uint32_t *skey = reinterpret_cast<uint32_t *>(ws + l.skey);
   uint32_t *sidx = reinterpret_cast<uint32_t *>(ws + l.sidx);
   uint32_t *tkey = reinterpret_cast<uint32_t *>(ws + l.tkey);
   uint32_t *tidx = reinterpret_cast<uint32_t *>(ws + l.tidx);
   uint32_t *shist = reinterpret_cast<uint32_t *>(ws + l.shist);
-  if (k > radix::kRankMax) {
-    // radix path: the last digit's scatter writes values_out / indices_out itself
-    const EmitSorted fin{priorities, values_out, indices_out, (uint32_t)n};
-    return radix::sort_pairs<uint32_t, uint32_t, EmitSorted>(ckey, skey, cidx, sidx, tkey, tidx, k,
-                                                             0, 32, shist, st, fin);
-  }
-  int rc = radix::sort_pairs<uint32_t, uint32_t>(ckey, skey, cidx, sidx, tkey, tidx, k, 0, 32,
-                                                 shist, st);
-  if (rc) return rc;
-  emit_kernel<<<dim3((unsigned)ceil_div64(k, kBlock)), block, 0, st>>>(priorities, sidx, k, n,
-                                                                      values_out, indices_out);
-  GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  return 0;
+  // the last digit's scatter writes values_out / indices_out itself
+  const EmitSorted fin{priorities, values_out, indices_out, (uint32_t)n};
+  return radix::sort_pairs<uint32_t, uint32_t, EmitSorted>(ckey, skey, cidx, sidx, tkey, tidx, k, 0,
+                                                           32, shist, st, fin);
 }

@@ -103,6 +103,57 @@ def test_topk_nan_priorities_stay_inside_the_outputs():
             assert bool((vals[k:] == -7.0).all()) and bool((idx[k:] == -7).all())
 
 
+def test_topk_value_order_paths(oracle):
+    """Value order: large groups of equal priorities above the threshold (the segment sort goes
+    down to the index bits), both sides of the k at which the radix sort takes over, and both
+    sides of the input size from which a sample is drawn."""
+    from gear_amd import ops
+    rng = np.random.default_rng(81)
+    ln = lambda n: (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    ties = ln(2_000_000)
+    ties[rng.permutation(2_000_000)[:60_000]] = 100.0
+    _check_topk(oracle, ops, ties, 65_536, "60 000 equal priorities above the threshold")
+    _check_topk(oracle, ops, ties, 50_000, "threshold inside the equal priorities")
+    three = rng.integers(0, 3, size=1_500_000).astype(np.float32)
+    _check_topk(oracle, ops, three, 131_072, "three distinct values, k = 131072")
+    big = ln(3_000_000)
+    _check_topk(oracle, ops, big, 131_072, "largest k of the segment sort")
+    _check_topk(oracle, ops, big, 131_073, "smallest k of the radix sort")
+    _check_topk(oracle, ops, ln(262_144), 1_000, "smallest input with a sample")
+    _check_topk(oracle, ops, ln(262_143), 1_000, "largest input without a sample")
+    _check_topk(oracle, ops, ln(30_000_000), 65_536, "long input")
+    wide = (rng.normal(size=1_000_000) * np.exp(rng.normal(size=1_000_000) * 8)).astype(np.float32)
+    _check_topk(oracle, ops, wide, 40_000, "priorities over many orders of magnitude, both signs")
+
+
+def _sampled_positions(n, samples=2048):
+    """Where the selection looks for its sample: one position per stride, at a hashed offset."""
+    stride = n // samples
+    s = np.arange(samples, dtype=np.uint64)
+    off = (((s * np.uint64(2654435761)) & np.uint64(0xffffffff)) * np.uint64(stride)) >> np.uint64(32)
+    return (s * np.uint64(stride) + off).astype(np.int64)
+
+
+def test_topk_with_a_misleading_sample(oracle):
+    """The sample only decides how the work is done: when it overstates the priorities (too few
+    candidates: the first read is done again on uniform bins) or understates them (every entry a
+    candidate: the lists overflow and the levels stream), the result is the same."""
+    from gear_amd import ops
+    rng = np.random.default_rng(71)
+    n = 2_000_000
+    base = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    pos = _sampled_positions(n)
+    high = base.copy()
+    high[pos] = 1000.0 + rng.random(pos.size, dtype=np.float32)
+    _check_topk(oracle, ops, high, 65_536, "sample overstates (redo)")
+    _check_topk(oracle, ops, high, 1_000, "sample overstates, k below the sampled entries")
+    low = base.copy()
+    low[pos] = 1e-6
+    _check_topk(oracle, ops, low, 65_536, "sample understates (lists overflow)")
+    neg = -base
+    _check_topk(oracle, ops, neg, 30_000, "all negative")
+
+
 def test_topk_config5_size(oracle):
     """Config 5's maintenance step at full size: top-65 536 of 10 000 000 lognormal^0.6."""
     from gear_amd import ops
