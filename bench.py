@@ -223,7 +223,11 @@ def run_config4(args):
                      "avg_launch_ms": gather_ms, "launch_ms_p10_p50_p90": [pct(0.1), pct(0.5), pct(0.9)],
                      "algorithmic_bytes": alg_bytes,
                      "traffic": args.traffic_bytes if args.traffic_bytes is not None else
-                     (MEASURED_GATHER_TRAFFIC_BYTES if cap == 1000 else None)},
+                     (MEASURED_GATHER_TRAFFIC_BYTES if cap == 1000 else None),
+                     "traffic_source": "--traffic-bytes" if args.traffic_bytes is not None else
+                     ("profiles/subcopy_multi_kernel_config4_hbm_traffic.txt (rocprofv3 --pmc "
+                      "FETCH_SIZE and WRITE_SIZE of this command, scaled by a 1 GiB copy; not "
+                      "re-measured in this run)" if cap == 1000 else None)},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst)
@@ -243,8 +247,8 @@ def cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst):
     def one_step(threads):
         u01 = rng.random(B, dtype=np.float32)
         t0 = time.perf_counter()
-        prefix = orc.scan_f32_f64(pri)
-        flat = orc.upper_bound_f64(prefix, u01, unit_uniforms=True)
+        prefix = orc.scan_f32_f64(pri, threads=threads)
+        flat = orc.upper_bound_f64(prefix, u01, unit_uniforms=True, threads=threads)
         flat = orc.sort_i64(flat)
         idxs = (flat // T) % keep
         tss = flat % T
@@ -263,8 +267,9 @@ def cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst):
         return nrun, t_total
 
     nrun, t_total = timed(1, 10.0)
-    # the gather over the host's share of cores (windows split over threads; scan, search and sort
-    # stay sequential): 16 threads at most, the CPU share of a one-GPU box
+    # the same step over the host's share of cores (two-level chunked scan, draws and windows split
+    # over threads; the sort of 2048 keys stays sequential): 16 threads at most, the CPU share of a
+    # one-GPU box
     cores = max(1, min(16, os.cpu_count() or 1))
     one_step(cores)
     nrun_mt, t_mt = timed(cores, 5.0)
@@ -276,8 +281,8 @@ def cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst):
             "sample": "%d steps of the same pipeline (fp64 scan of 1e6 priorities, 2048 searches, "
                       "sort, 4-column gather with memset+memcpy per window) on the first %d of %d "
                       "trajectories (%.1f GB of the table, trajectory index taken modulo %d); "
-                      "host has %d logical cores; value uses 1, all_cores splits the gather's "
-                      "windows over %d threads (%d steps)"
+                      "host has %d logical cores; value uses 1, all_cores runs a chunked scan and "
+                      "splits draws and windows over %d threads (%d steps)"
                       % (nrun, keep, tab.capacity, keep * tab.traj_stride / 1e9, keep,
                          os.cpu_count() or 0, cores, nrun_mt)}
 
@@ -468,9 +473,9 @@ def run_config2(args):
         k += 1
     cpu_ms = (time.perf_counter() - t0) * 1e3 / k
     return _line(B / (ms * 1e-3), "draws/s", args, ms,
-                 "config2: 1e6 fp32 priorities -> fp64 prefix (init + scan kernels), 4096 draws, "
-                 "importance weights",
-                 {"bound": "hbm", "kernel": "scan_init_kernel + scan_kernel", "achieved": alg / (sms * 1e-3) / 1e9,
+                 "config2: 1e6 fp32 priorities -> fp64 prefix (one chained single-pass launch), 4096 "
+                 "draws, importance weights",
+                 {"bound": "hbm", "kernel": "scan_ranges_kernel<float, double, 4, NR, true>", "achieved": alg / (sms * 1e-3) / 1e9,
                   "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (sms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                   "avg_launch_ms": sms, "algorithmic_bytes": alg, "traffic": None},
                  dict(_graph_extra(B, "draws/s", ms_graph),
@@ -686,9 +691,40 @@ def run_config5(args):
                 parts_cpu[n_] += d_ * 1e3
             nrun += 1
         cpu_ms = (time.perf_counter() - t_all) * 1e3 / nrun
+        # the same step over the host's share of cores: per-chunk top-k selection + merge, two-level
+        # chunked scan, draws and windows split over threads (scatter and the 2048-key sort stay
+        # sequential)
+        cores = max(1, min(16, os.cpu_count() or 1))
+        parts_mt = {n: 0.0 for n in names}
+        t_mt = time.perf_counter()
+        nmt = 0
+        while nmt < 2 or (time.perf_counter() - t_mt < 6.0 and nmt < 40):
+            t0 = time.perf_counter()
+            orc.scatter_f32(hp, hidx[nmt % 4], hval[nmt % 4])
+            t1 = time.perf_counter()
+            orc.topk_f32(hp, k, True, threads=cores)
+            t2 = time.perf_counter()
+            pre = orc.scan_f32_f64(hp, threads=cores)
+            t3 = time.perf_counter()
+            fl = orc.sort_i64(orc.upper_bound_f64(pre, crng.random(B, dtype=np.float32),
+                                                  unit_uniforms=True, threads=cores)) % (T * cap)
+            t4 = time.perf_counter()
+            for c in range(4):
+                orc.subcopy(host, (fl // T) % keep, fl % T, fl % T + 1, True, ofst, span,
+                            tab.traj_stride, tab.step_bytes[c], tab.col_base(c), dst=hd[c],
+                            threads=cores)
+            t5 = time.perf_counter()
+            for n_, d_ in zip(names, (t1 - t0, t2 - t1, t3 - t2, t4 - t3, t5 - t4)):
+                parts_mt[n_] += d_ * 1e3
+            nmt += 1
+        mt_ms = (time.perf_counter() - t_mt) * 1e3 / nmt
         extra5["cpu_baseline"] = {
             "value": B / (cpu_ms * 1e-3), "unit": "windows/s", "cores": 1, "kind": "port",
             "ms_per_step": cpu_ms, "parts_ms": {n_: v / nrun for n_, v in parts_cpu.items()},
+            "all_cores": {"value": B / (mt_ms * 1e-3), "unit": "windows/s", "cores": cores,
+                          "ms_per_step": mt_ms, "steps": nmt,
+                          "parts_ms": {n_: v / nmt for n_, v in parts_mt.items()}},
+            "cpu_model": cpu_model(),
             "sample": "%d steps: scatter 65536, top-65536 of 1e7, fp64 rescan of 1e7, 2048 draws, "
                       "4-column gather from the first %d trajectories of the host table"
                       % (nrun, keep)}

@@ -158,6 +158,38 @@ ORACLE_API void oracle_scan_i64(const int64_t *in, int64_t *out, int64_t n) {
   }
 }
 
+/* The same prefix sum over `threads` host threads: every thread sums a contiguous chunk, the
+ * chunk sums are scanned sequentially, every thread then scans its chunk from its offset.  Only
+ * the all-cores leg of the CPU baseline uses it.  The summation order differs from the
+ * sequential scan's, so results agree to rounding (exactly on integer-valued input; tested). */
+ORACLE_API void oracle_scan_f32_f64_mt(const float *in, double *out, int64_t n, int threads) {
+  if (threads < 1) threads = 1;
+  if (threads > 256) threads = 256;
+  double sums[256];
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int t = 0; t < threads; ++t) {
+    const int64_t lo = n * t / threads, hi = n * (t + 1) / threads;
+    double acc = 0.0;
+    for (int64_t i = lo; i < hi; ++i) acc += (double)in[i];
+    sums[t] = acc;
+  }
+  double run = 0.0;
+  for (int t = 0; t < threads; ++t) {
+    const double s = sums[t];
+    sums[t] = run;
+    run += s;
+  }
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int t = 0; t < threads; ++t) {
+    const int64_t lo = n * t / threads, hi = n * (t + 1) / threads;
+    double acc = sums[t];
+    for (int64_t i = lo; i < hi; ++i) {
+      acc += (double)in[i];
+      out[i] = acc;
+    }
+  }
+}
+
 /* Sum of fp32 values (src/cuda/one_dim_sum.cu:22-74 computes it with fp32 atomics); here the
  * sequential fp64 sum, rounded once to fp32. */
 ORACLE_API double oracle_sum_f32(const float *in, int64_t n) {
@@ -188,6 +220,18 @@ ORACLE_API void oracle_upper_bound_f64(const double *prefix, int64_t n, const fl
     int64_t i = upper_bound_f64(prefix, n, t);
     if (i > n - 1) i = n - 1;
     idx_out[j] = i;
+  }
+}
+
+/* The same search with the draws split over `threads` host threads (identical results). */
+ORACLE_API void oracle_upper_bound_f64_mt(const double *prefix, int64_t n, const float *u,
+                                          int64_t num, int unit_uniforms, int64_t *idx_out,
+                                          int threads) {
+  if (threads < 1) threads = 1;
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int t = 0; t < threads; ++t) {
+    const int64_t lo = num * t / threads, hi = num * (t + 1) / threads;
+    if (hi > lo) oracle_upper_bound_f64(prefix, n, u + lo, hi - lo, unit_uniforms, idx_out + lo);
   }
 }
 
@@ -248,16 +292,9 @@ static int cmp_i64(const void *a, const void *b) {
 }
 
 /* Keeps a k-sized candidate set by quickselect on (value desc, index asc), then orders it. */
-ORACLE_API void oracle_topk_f32(const float *w, int64_t n, int64_t k, int sorted_by_value,
-                                float *values_out, int64_t *indices_out) {
-  if (k <= 0 || n <= 0) return;
-  if (k > n) k = n;
-  oracle_vi *a = (oracle_vi *)malloc(sizeof(oracle_vi) * (size_t)n);
-  for (int64_t i = 0; i < n; ++i) {
-    a[i].v = w[i];
-    a[i].i = i;
-  }
-  /* quickselect: after the loop a[0..k) holds the k first elements of the total order */
+/* a[0, k) becomes the k first elements of the total order (value descending, index ascending),
+ * sorted: quickselect with a seeded pivot sequence, then qsort of the front. */
+static void select_front(oracle_vi *a, int64_t n, int64_t k) {
   int64_t lo = 0, hi = n - 1;
   uint64_t rng = 0x9E3779B97F4A7C15ull;
   while (lo < hi) {
@@ -286,6 +323,10 @@ ORACLE_API void oracle_topk_f32(const float *w, int64_t n, int64_t k, int sorted
       break;
   }
   qsort(a, (size_t)k, sizeof(oracle_vi), cmp_desc_stable);
+}
+
+static void topk_emit(const float *w, const oracle_vi *a, int64_t k, int sorted_by_value,
+                      float *values_out, int64_t *indices_out) {
   if (sorted_by_value) {
     for (int64_t j = 0; j < k; ++j) {
       if (values_out) values_out[j] = a[j].v;
@@ -297,10 +338,56 @@ ORACLE_API void oracle_topk_f32(const float *w, int64_t n, int64_t k, int sorted
     if (values_out)
       for (int64_t j = 0; j < k; ++j) values_out[j] = w[indices_out[j]];
   }
+}
+
+ORACLE_API void oracle_topk_f32(const float *w, int64_t n, int64_t k, int sorted_by_value,
+                                float *values_out, int64_t *indices_out) {
+  if (k <= 0 || n <= 0) return;
+  if (k > n) k = n;
+  oracle_vi *a = (oracle_vi *)malloc(sizeof(oracle_vi) * (size_t)n);
+  for (int64_t i = 0; i < n; ++i) {
+    a[i].v = w[i];
+    a[i].i = i;
+  }
+  select_front(a, n, k);
+  topk_emit(w, a, k, sorted_by_value, values_out, indices_out);
   free(a);
 }
 
-/* ---- sort of sampled indices: torch.sort(...).values of global_sampler.py:131,172,195 ------- */
+/* The same selection over `threads` host threads: every thread selects the top min(k, chunk)
+ * of a contiguous chunk, the survivors (at most threads * k) go through one more selection.
+ * Only the all-cores leg of the CPU baseline uses it; the result is identical to
+ * oracle_topk_f32 (the total order is the same; tested). */
+ORACLE_API void oracle_topk_f32_mt(const float *w, int64_t n, int64_t k, int sorted_by_value,
+                                   float *values_out, int64_t *indices_out, int threads) {
+  if (k <= 0 || n <= 0) return;
+  if (k > n) k = n;
+  if (threads < 1) threads = 1;
+  if (threads > 256) threads = 256;
+  oracle_vi *a = (oracle_vi *)malloc(sizeof(oracle_vi) * (size_t)n);
+  int64_t kept[256];
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int t = 0; t < threads; ++t) {
+    const int64_t lo = n * t / threads, hi = n * (t + 1) / threads;
+    for (int64_t i = lo; i < hi; ++i) {
+      a[i].v = w[i];
+      a[i].i = i;
+    }
+    const int64_t kk = k < hi - lo ? k : hi - lo;
+    if (kk > 0) select_front(a + lo, hi - lo, kk);
+    kept[t] = kk;
+  }
+  int64_t m = 0;
+  for (int t = 0; t < threads; ++t) {
+    const int64_t lo = n * t / threads;
+    if (lo != m) memmove(a + m, a + lo, sizeof(oracle_vi) * (size_t)kept[t]);
+    m += kept[t];
+  }
+  select_front(a, m, k);
+  topk_emit(w, a, k, sorted_by_value, values_out, indices_out);
+  free(a);
+}
+
 typedef struct {
   int64_t k;
   int64_t pos;

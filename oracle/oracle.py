@@ -108,10 +108,16 @@ def copy(src, dst, src_offsets, dst_offsets, stride):
     return dst
 
 
-def scan_f32_f64(p):
+def scan_f32_f64(p, threads=1):
+    """threads > 1: two-level chunked scan over that many host threads (all-cores baseline);
+    equal to the sequential result up to rounding, exactly on integer-valued input."""
     p = _c(p, np.float32)
     out = np.zeros(len(p), np.float64)
-    lib().oracle_scan_f32_f64(_p(p, _f32p), _p(out, _f64p), ctypes.c_int64(len(p)))
+    if threads > 1:
+        lib().oracle_scan_f32_f64_mt(_p(p, _f32p), _p(out, _f64p), ctypes.c_int64(len(p)),
+                                     ctypes.c_int(int(threads)))
+    else:
+        lib().oracle_scan_f32_f64(_p(p, _f32p), _p(out, _f64p), ctypes.c_int64(len(p)))
     return out
 
 
@@ -127,12 +133,15 @@ def sum_f32(p):
     return lib().oracle_sum_f32(_p(p, _f32p), ctypes.c_int64(len(p)))
 
 
-def upper_bound_f64(prefix, u, unit_uniforms=False):
+def upper_bound_f64(prefix, u, unit_uniforms=False, threads=1):
     prefix, u = _c(prefix, np.float64), _c(u, np.float32)
     out = np.zeros(len(u), np.int64)
-    lib().oracle_upper_bound_f64(_p(prefix, _f64p), ctypes.c_int64(len(prefix)), _p(u, _f32p),
-                                 ctypes.c_int64(len(u)), ctypes.c_int(int(unit_uniforms)),
-                                 _p(out, _i64p))
+    args = [_p(prefix, _f64p), ctypes.c_int64(len(prefix)), _p(u, _f32p),
+            ctypes.c_int64(len(u)), ctypes.c_int(int(unit_uniforms)), _p(out, _i64p)]
+    if threads > 1:
+        lib().oracle_upper_bound_f64_mt(*args, ctypes.c_int(int(threads)))
+    else:
+        lib().oracle_upper_bound_f64(*args)
     return out
 
 
@@ -155,12 +164,18 @@ def is_weights(priorities, total, idx, beta):
     return out
 
 
-def topk_f32(w, k, sorted_by_value=True):
+def topk_f32(w, k, sorted_by_value=True, threads=1):
+    """threads > 1: per-chunk selection over that many host threads, then a merge (all-cores
+    baseline); identical result."""
     w = _c(w, np.float32)
     vals = np.zeros(k, np.float32)
     idx = np.zeros(k, np.int64)
-    lib().oracle_topk_f32(_p(w, _f32p), ctypes.c_int64(len(w)), ctypes.c_int64(k),
-                          ctypes.c_int(int(sorted_by_value)), _p(vals, _f32p), _p(idx, _i64p))
+    args = [_p(w, _f32p), ctypes.c_int64(len(w)), ctypes.c_int64(k),
+            ctypes.c_int(int(sorted_by_value)), _p(vals, _f32p), _p(idx, _i64p)]
+    if threads > 1:
+        lib().oracle_topk_f32_mt(*args, ctypes.c_int(int(threads)))
+    else:
+        lib().oracle_topk_f32(*args)
     return vals, idx
 
 

@@ -111,3 +111,27 @@ def test_scatter_last_wins(oracle, fx):
     w = np.zeros(4, np.float32)
     oracle.scatter_f32(w, [1, 1, 3, 1, 9, -1], np.array([1, 2, 3, 4, 5, 6], np.float32))
     assert list(w) == [0, 4, 0, 3]
+
+
+@pytest.mark.parametrize("threads", [2, 3, 8])
+def test_multithreaded_baselines_equal_the_sequential_oracle(oracle, threads):
+    """The all-cores legs of the CPU baseline (chunked scan, per-chunk top-k + merge, draws split
+    over threads) against the single-threaded functions they stand beside."""
+    rng = np.random.default_rng(threads)
+    ints = rng.integers(0, 1000, size=100_003).astype(np.float32)
+    assert np.array_equal(oracle.scan_f32_f64(ints, threads=threads), np.cumsum(ints.astype(np.float64)))
+    p = (rng.lognormal(0, 1, size=100_003) ** 0.6).astype(np.float32)
+    seq = oracle.scan_f32_f64(p)
+    par = oracle.scan_f32_f64(p, threads=threads)
+    assert np.max(np.abs(par - seq) / seq) <= 1e-13
+    u = rng.random(1000, dtype=np.float32)
+    assert np.array_equal(oracle.upper_bound_f64(seq, u, True, threads=threads),
+                          oracle.upper_bound_f64(seq, u, True))
+    w = rng.integers(0, 50, size=50_001).astype(np.float32)        # many ties
+    for k in (1, 777, 50_001):
+        for by_value in (True, False):
+            a = oracle.topk_f32(w, k, by_value)
+            b = oracle.topk_f32(w, k, by_value, threads=threads)
+            assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    assert np.array_equal(oracle.topk_f32(w, 777, True, threads=threads)[1],
+                          np.argsort(-w.astype(np.float64), kind="stable")[:777])
