@@ -744,6 +744,91 @@ def run_config5(args):
                                    "rescan_GBps": 12 * npri / (parts["scan"] * 1e-3) / 1e9}))
 
 
+def _calibrate_copy(torch, ops):
+    """Three plain 1 GiB copies through the library's slice kernel: the launch of known size that
+    the FETCH_SIZE / WRITE_SIZE counters of the other kernels in the same run are scaled by."""
+    nb = 1 << 30
+    csrc = torch.zeros(nb, dtype=torch.uint8, device="cuda")
+    cdst = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    zero = torch.zeros(1, dtype=torch.int64, device="cuda")
+    for _ in range(3):
+        ops.copy(csrc, cdst, zero, zero, nb)
+    torch.cuda.synchronize()
+
+
+def run_scan(args):
+    """One kernel chain on its own: fp64 prefix sum of --n fp32 priorities.  The variant follows
+    GEAR_HIP_SCAN_SINGLE_PASS (unset or 1: chained single pass, 0: range sums + scan in two
+    launches, 2: ticketed look-back)."""
+    import numpy as np
+    import torch
+    from gear_amd import ops
+    n = args.n
+    rng = np.random.default_rng(7)
+    pri = torch.from_numpy((rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)).cuda()
+    prefix = torch.empty(n, dtype=torch.float64, device="cuda")
+    if args.calibrate_copy:
+        _calibrate_copy(torch, ops)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+
+    def step(i, slot):
+        if slot is not None:
+            ev[slot][0].record()
+        ops.prefix_sum(pri, out=prefix)
+        if slot is not None:
+            ev[slot][1].record()
+
+    ms = _time_steps(torch, step, args.steps, args.warmup)
+    sms = sorted(a.elapsed_time(b) for a, b in ev)
+    avg = sum(sms) / len(sms)
+    alg = 12 * n
+    variant = {"": "chained single pass (default)", "1": "chained single pass", "0": "two launches",
+               "2": "ticketed look-back"}.get(os.environ.get("GEAR_HIP_SCAN_SINGLE_PASS", ""), "?")
+    return _line(n / (ms * 1e-3), "priorities/s", args, ms,
+                 "scan: fp64 prefix sum of %d fp32 priorities, %s" % (n, variant),
+                 {"bound": "hbm", "kernel": "prefix sum chain (" + variant + ")",
+                  "achieved": alg / (avg * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                  "frac": alg / (avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, "avg_launch_ms": avg,
+                  "median_launch_ms": sms[len(sms) // 2], "algorithmic_bytes": alg,
+                  "traffic": None})
+
+
+def run_topk(args):
+    """One kernel chain on its own: top --k of --n fp32 priorities (--topk-order value|index)."""
+    import numpy as np
+    import torch
+    from gear_amd import ops
+    n, k = args.n, args.k
+    by_value = args.topk_order == "value"
+    rng = np.random.default_rng(7)
+    pri = torch.from_numpy((rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)).cuda()
+    if args.calibrate_copy:
+        _calibrate_copy(torch, ops)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+
+    def step(i, slot):
+        if slot is not None:
+            ev[slot][0].record()
+        ops.topk(pri, k, sorted_by_value=by_value)
+        if slot is not None:
+            ev[slot][1].record()
+
+    ms = _time_steps(torch, step, args.steps, args.warmup)
+    sms = sorted(a.elapsed_time(b) for a, b in ev)
+    avg = sum(sms) / len(sms)
+    alg = 4 * n + 12 * k
+    return _line(n / (ms * 1e-3), "priorities/s", args, ms,
+                 "topk: top %d of %d fp32 priorities, ordered by %s" % (k, n, args.topk_order),
+                 {"bound": "hbm", "kernel": "top-k chain (prep, level0, member_hist x2, count, "
+                                            "write" + (", segment_sort)" if by_value else ")"),
+                  "achieved": alg / (avg * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                  "frac": alg / (avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, "avg_launch_ms": avg,
+                  "median_launch_ms": sms[len(sms) // 2], "algorithmic_bytes": alg,
+                  "traffic": None})
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -752,8 +837,12 @@ def main():
     ap.add_argument("--trajectories", type=int, default=1000,
                     help="config 4: trajectories of 1000 steps in the table (1000 = full size)")
     ap.add_argument("--workload", default="config4",
-                    choices=["config1", "config2", "config3", "config4", "config5"],
-                    help="BASELINE config to run (config4 is the bench line)")
+                    choices=["config1", "config2", "config3", "config4", "config5", "scan", "topk"],
+                    help="BASELINE config to run (config4 is the bench line); scan and topk run "
+                         "one maintenance kernel chain on its own, for profiles")
+    ap.add_argument("--n", type=int, default=10_000_000, help="scan / topk: number of priorities")
+    ap.add_argument("--k", type=int, default=65_536, help="topk: entries kept")
+    ap.add_argument("--topk-order", default="value", choices=["value", "index"])
     ap.add_argument("--trajectories3", type=int, default=100_000,
                     help="config 3: number of trajectories (100000 = full size, 10.4 GB)")
     ap.add_argument("--trajectories5", type=int, default=2000,
@@ -771,7 +860,8 @@ def main():
               % args.gpus, file=sys.stderr)
         sys.exit(2)
     runner = {"config1": run_config1, "config2": run_config2, "config3": run_config3,
-              "config4": run_config4, "config5": run_config5}[args.workload]
+              "config4": run_config4, "config5": run_config5, "scan": run_scan,
+              "topk": run_topk}[args.workload]
     result = runner(args)
     print(json.dumps(result), flush=True)
 

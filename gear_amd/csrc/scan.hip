@@ -1,9 +1,10 @@
 // Inclusive prefix sums and a deterministic sum, gfx950.  fp32 inputs are accumulated in fp64.
 //
-// Three kernels share the inner scan (each thread scans inside its 16-byte input vectors, row sums
-// go through a DPP wave scan, wave totals meet in LDS, results leave through LDS so that every store
-// instruction writes whole lines):
-//  * chained single pass, up to 2048 ranges: scan_ranges_kernel<CHAINED = true>.  A workgroup
+// The range kernels work on blocked ranges: thread t of a workgroup owns G consecutive 16-byte
+// granules of its range, adds them up in order, and one DPP wave scan per range joins the
+// threads (a wave-private LDS row turns the row-major order of the memory instructions, 1 KiB of
+// consecutive addresses per wave and instruction, into that blocked order and back):
+//  * chained single pass, up to 4096 ranges: scan_ranges_kernel<CHAINED = true>.  A workgroup
 //    keeps its range in registers, publishes the range's sum and adds the sums of ALL earlier
 //    ranges (fixed order: bit-reproducible), then writes the prefix: the input is read once.
 //    Range r belongs to workgroup r (no ticket).  A published sum travels as three 64-bit words
@@ -11,9 +12,9 @@
 //    on its own: no fence, no flag, nothing to clear before a call (a host counter hands every
 //    call a fresh tag; what an earlier call or an uninitialised workspace left never matches).
 //    The wait for a predecessor is bounded: when it runs out, the workgroup sums that
-//    predecessor's range itself, with the same reduction tree, so no kernel can spin forever and
-//    the result does not change.
-//  * two launches, up to 8192 ranges (n <= 134 M fp32): range_sum_kernel writes the sum of every
+//    predecessor's range itself, with the same reduction tree, and publishes it on the
+//    predecessor's behalf, so no kernel can spin forever and the result does not change.
+//  * two launches, up to 16384 ranges (n <= 134 M fp32): range_sum_kernel writes the sum of every
 //    range; scan_ranges_kernel<CHAINED = false> re-reads its range (now in L2 / MALL), adds the
 //    sums of all earlier ranges and writes the prefix.  No workgroup waits for another one.  Used
 //    for long inputs, under stream capture (a captured launch would replay its tag) and for the
@@ -239,8 +240,8 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
 // sum of ALL earlier ranges' sums (each thread adds its share of them, fixed summation order).
 // Nobody waits for an inclusive value, so there is no serial chain across the XCDs, and the result
 // is bit-reproducible from run to run.
-constexpr int kMaxRanges = 2048;     // chained: every thread polls up to 8 range sums
-constexpr int kMaxRangesTwo = 8192;  // two launches: every thread adds up to 32 range sums
+constexpr int kMaxRanges = 4096;      // chained: every thread polls up to 16 range sums
+constexpr int kMaxRangesTwo = 16384;  // two launches: every thread adds up to 64 range sums
 
 // A range sum in flight between workgroups of one launch: three self-validating words.
 constexpr int kTagBits = 42;
@@ -259,36 +260,140 @@ __device__ __forceinline__ bool try_read(const Slot *s, uint64_t tag, uint64_t *
   return (a >> 22) == tag && (b >> 22) == tag && (c >> 22) == tag;
 }
 
-// The sum of one range with the reduction tree every kernel here uses for it (thread: rows in
-// order, vector elements in order; wave: DPP tree; workgroup: (w0 + w1) + (w2 + w3)), returned to
-// every thread.  `red` is LDS for the four wave sums; the caller separates calls with a barrier.
-template <typename In, typename Acc, int VE, int NR>
+// ---- blocked ranges -------------------------------------------------------------------------------
+// A range is 256 threads x G granules of 16 bytes; thread t owns the G consecutive granules
+// [t*G, t*G + G) of its range (EPT = G * 16 / sizeof(In) consecutive elements), so that one serial
+// pass over registers and ONE wave scan per range replace a wave scan per row.  Global loads and
+// stores stay contiguous per instruction (1 KiB per wave): a wave-private LDS row turns the
+// row-major order of the memory instructions into the blocked order of the arithmetic and back.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <typename T> struct Gran {  // one 16-byte granule of T
+  static constexpr int kN = 16 / (int)sizeof(T);
+  typedef T type __attribute__((ext_vector_type(kN)));
+  typedef T loose __attribute__((ext_vector_type(kN), aligned(sizeof(T))));
+};
+
+template <typename In, typename Out, int G> struct Geo {
+  static constexpr int kVE = Gran<In>::kN;
+  static constexpr int kEPT = G * kVE;                       // elements per thread
+  static constexpr int kRange = kBlock * kEPT;               // elements per range
+  static constexpr int kWaveElems = kWave * kEPT;
+  static constexpr int kOE = Gran<Out>::kN;
+  static constexpr int kOG = kEPT / kOE;                     // result granules per thread
+  static constexpr int kPiece = kOG <= G ? kWave : kWave * G / kOG;  // lanes per store piece
+  static constexpr int kPitchIn = G + 1, kPitchOut = kOG + 1;  // odd pitches: no bank conflicts
+  static constexpr int kStage = kWave * kPitchIn;            // granules of LDS per wave
+  static_assert(kPiece * kPitchOut <= kStage, "result piece fits the staging row");
+  static_assert((G & (G - 1)) == 0 && (kOG & (kOG - 1)) == 0, "powers of two");
+};
+
+// The wave's kWaveElems elements starting at wbase, in blocked order: f[] of lane l holds elements
+// [wbase + l*EPT, wbase + (l+1)*EPT); elements at or beyond n read as 0.
+template <typename In, typename Out, int G>
+__device__ __forceinline__ void load_blocked(const In *__restrict__ in, int64_t n, int64_t wbase,
+                                             u32x4 *stage, int lane,
+                                             In (&f)[Geo<In, Out, G>::kEPT]) {
+  typedef Geo<In, Out, G> geo;
+  typedef typename Gran<In>::loose in_vec;
+  typedef typename Gran<In>::type in_gran;
+  if (wbase + geo::kWaveElems <= n) {
+    in_vec v[G];
+#pragma unroll
+    for (int r = 0; r < G; ++r)
+      v[r] = __builtin_nontemporal_load(
+          reinterpret_cast<const in_vec *>(in + wbase + (int64_t)(r * kWave + lane) * geo::kVE));
+#pragma unroll
+    for (int r = 0; r < G; ++r) {
+      const int g = r * kWave + lane;
+      in_gran q;
+#pragma unroll
+      for (int k = 0; k < geo::kVE; ++k) q[k] = v[r][k];
+      stage[(g / G) * geo::kPitchIn + (g % G)] = __builtin_bit_cast(u32x4, q);
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < G; ++r) {
+      const int g = r * kWave + lane;
+      const int64_t e0 = wbase + (int64_t)g * geo::kVE;
+      in_gran q;
+#pragma unroll
+      for (int k = 0; k < geo::kVE; ++k) q[k] = (e0 + k < n) ? in[e0 + k] : (In)0;
+      stage[(g / G) * geo::kPitchIn + (g % G)] = __builtin_bit_cast(u32x4, q);
+    }
+  }
+  wave_lds_sync();
+#pragma unroll
+  for (int j = 0; j < G; ++j) {
+    const in_gran q = __builtin_bit_cast(in_gran, stage[lane * geo::kPitchIn + j]);
+#pragma unroll
+    for (int k = 0; k < geo::kVE; ++k) f[j * geo::kVE + k] = q[k];
+  }
+  wave_lds_sync();
+}
+
+// Sum of a thread's elements in order, then the wave's inclusive scan of those sums.
+template <typename In, typename Acc, int EPT>
+__device__ __forceinline__ Acc thread_total(const In (&f)[EPT]) {
+  Acc t = (Acc)f[0];
+#pragma unroll
+  for (int e = 1; e < EPT; ++e) t += (Acc)f[e];
+  return t;
+}
+
+// The sum of one range with the reduction tree every kernel here uses for it (thread: its
+// elements in order; wave: the DPP scan's last lane; workgroup: (w0 + w1) + (w2 + w3)), returned
+// to every thread.  `red` is LDS for the four wave sums; the caller separates calls with a barrier.
+template <typename In, typename Acc, typename Out, int G>
 __device__ __forceinline__ Acc range_total(const In *__restrict__ in, int64_t n, int64_t range,
-                                           Acc *red) {
-  constexpr int kElems = NR * kBlock * VE;
-  typedef typename InVec<In, VE>::type in_vec;
+                                           u32x4 *stage, Acc *red) {
+  typedef Geo<In, Out, G> geo;
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-  const int64_t base = range * kElems;
-  Acc tsum = (Acc)0;
+  In f[geo::kEPT];
+  load_blocked<In, Out, G>(in, n, range * geo::kRange + (int64_t)wave * geo::kWaveElems, stage, lane,
+                           f);
+  const Acc inc = wave_inclusive_sum(thread_total<In, Acc, geo::kEPT>(f));
+  if (lane == kWave - 1) red[wave] = inc;
+  __syncthreads();
+  const Acc total = (red[0] + red[1]) + (red[2] + red[3]);
+  __syncthreads();
+  return total;
+}
+
+// The same sum with the same tree, read straight from memory (a lane's elements are consecutive,
+// so its loads do not share lines with its neighbours': slow, and light on registers).  For the
+// rare workgroup that has to add up a predecessor's range while its own is in registers.
+template <typename In, typename Acc, typename Out, int G>
+__device__ __noinline__ Acc range_total_direct(const In *__restrict__ in, int64_t n, int64_t range,
+                                               Acc *red) {
+  typedef Geo<In, Out, G> geo;
+  typedef typename Gran<In>::loose in_vec;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  const int64_t e0 = range * geo::kRange + (int64_t)tid * geo::kEPT;
+  Acc t = (Acc)0;
+#pragma unroll 1
+  for (int j = 0; j < G; ++j) {
+    const int64_t e = e0 + (int64_t)j * geo::kVE;
+    In q[geo::kVE];
+    if (e + geo::kVE <= n) {
+      const in_vec v = *reinterpret_cast<const in_vec *>(in + e);
 #pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
-    In raw[VE];
-    if (e0 + VE <= n) {
-      const in_vec v = *reinterpret_cast<const in_vec *>(in + e0);
-#pragma unroll
-      for (int j = 0; j < VE; ++j) raw[j] = v[j];
+      for (int k = 0; k < geo::kVE; ++k) q[k] = v[k];
     } else {
 #pragma unroll
-      for (int j = 0; j < VE; ++j) raw[j] = (e0 + j < n) ? in[e0 + j] : (In)0;
+      for (int k = 0; k < geo::kVE; ++k) q[k] = (e + k < n) ? in[e + k] : (In)0;
     }
-    Acc a = (Acc)raw[0];
 #pragma unroll
-    for (int j = 1; j < VE; ++j) a += (Acc)raw[j];
-    tsum += a;
+    for (int k = 0; k < geo::kVE; ++k) t = (j == 0 && k == 0) ? (Acc)q[0] : t + (Acc)q[k];
   }
-  const Acc w = wave_sum(tsum);
-  if (lane == 0) red[wave] = w;
+  const Acc inc = wave_inclusive_sum(t);
+  if (lane == kWave - 1) red[wave] = inc;
   __syncthreads();
   const Acc total = (red[0] + red[1]) + (red[2] + red[3]);
   __syncthreads();
@@ -297,13 +402,14 @@ __device__ __forceinline__ Acc range_total(const In *__restrict__ in, int64_t n,
 
 // Sum of every range, one workgroup per range: the first launch of the two-launch variant, in
 // which the scan launch below finds all sums ready (no publishing, no polling).
-template <typename In, typename Acc, int VE, int NR>
+template <typename In, typename Acc, typename Out, int G>
 __global__ __launch_bounds__(kBlock) void range_sum_kernel(const In *__restrict__ in, int64_t n,
                                                            uint64_t *__restrict__ sums,
                                                            int64_t first_range) {
+  __shared__ u32x4 stage[kBlock / kWave][Geo<In, Out, G>::kStage];
   __shared__ Acc red[kBlock / kWave];
   const int64_t range = first_range + blockIdx.x;
-  const Acc total = range_total<In, Acc, VE, NR>(in, n, range, red);
+  const Acc total = range_total<In, Acc, Out, G>(in, n, range, stage[threadIdx.x >> 6], red);
   if (threadIdx.x == 0) sums[range] = Bits<Acc>::to(total);
 }
 
@@ -312,148 +418,185 @@ __global__ __launch_bounds__(kBlock) void range_sum_kernel(const In *__restrict_
 // slots[r]  CHAINED only: the same sums as tagged words, for the workgroups of this launch
 // spin_limit  CHAINED only: polls of a missing predecessor before the workgroup sums that range
 //           itself
-template <typename In, typename Acc, typename Out, int VE, int NR, bool CHAINED>
+template <typename In, typename Acc, typename Out, int G, bool CHAINED>
 __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restrict__ in,
                                                              Out *__restrict__ out, int64_t n,
                                                              uint64_t *__restrict__ sums,
                                                              Slot *__restrict__ slots,
                                                              int64_t first_range, uint64_t tag,
                                                              int spin_limit) {
-  constexpr int kElems = NR * kBlock * VE;
+  typedef Geo<In, Out, G> geo;
+  typedef typename Gran<Out>::type out_gran;
   constexpr int kWaves = kBlock / kWave;
-  typedef typename InVec<In, VE>::type in_vec;
-  __shared__ Acc wtot[NR][kWaves];
-  __shared__ Out stage[kWaves][kWave * VE];
+  constexpr int kPolls = (CHAINED ? kMaxRanges : kMaxRangesTwo) / kBlock;
+  constexpr int kBatch = 4;
+  __shared__ u32x4 stage_all[kWaves][geo::kStage];
+  __shared__ Acc wtot[kWaves];
   __shared__ Acc red[kWaves];
-  __shared__ int s_missing;
-  __shared__ uint16_t s_queue[CHAINED ? kMaxRanges : 1];
+  __shared__ uint32_t s_missing[CHAINED ? kMaxRanges / 32 : 1];  // one bit per unpublished range
 
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
   const int64_t tile = first_range + (int64_t)blockIdx.x;
-  const int64_t base = tile * kElems;
+  const int64_t wbase = tile * geo::kRange + (int64_t)wave * geo::kWaveElems;
+  u32x4 *stage = stage_all[wave];
 
   if (CHAINED) {
-    if (tid == 0) s_missing = 0;
-    __syncthreads();
+    if (tid < kMaxRanges / 32) s_missing[tid] = 0u;
   }
-
-  In raw[NR][VE];
-  Acc s[NR];
-  Acc tsum = (Acc)0;
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
-    if (e0 + VE <= n) {
-      const in_vec v = __builtin_nontemporal_load(reinterpret_cast<const in_vec *>(in + e0));
-#pragma unroll
-      for (int j = 0; j < VE; ++j) raw[r][j] = v[j];
-    } else {
-#pragma unroll
-      for (int j = 0; j < VE; ++j) raw[r][j] = (e0 + j < n) ? in[e0 + j] : (In)0;
-    }
+  In f[geo::kEPT];
+  load_blocked<In, Out, G>(in, n, wbase, stage, lane, f);
+  const Acc inc = wave_inclusive_sum(thread_total<In, Acc, geo::kEPT>(f));
+  const Acc wexcl = wave_shift_up1(inc);
+  if (lane == kWave - 1) wtot[wave] = inc;
+  __syncthreads();
+  const Acc w0 = wtot[0], w1 = wtot[1], w2 = wtot[2], w3 = wtot[3];
+  // the range's sum goes out first
+  if (CHAINED && tid == 0) {
+    const uint64_t bits = Bits<Acc>::to((w0 + w1) + (w2 + w3));
+    publish(&slots[tile], tag, bits);
+    sums[tile] = bits;
   }
+  // Sum of every earlier range: thread t adds ranges t, t+256, ... in that order.  The ones
+  // before this launch's first range are plain words from an earlier call, the others are
+  // published by the workgroups of this launch.  They are read kBatch at a time (all polls of a
+  // batch are issued together, only the unpublished ones are repeated).  What is still missing
+  // after the bounded wait is summed by this workgroup from the input, with the tree its own
+  // workgroup uses, and published on its behalf (same bits): the kernel ends whatever the others
+  // do, and the next pass over the words finds everything.
+  Acc part = (Acc)0;
+  bool failed = CHAINED;
+  for (int attempt = 0; attempt < (CHAINED ? 3 : 1); ++attempt) {
+    part = (Acc)0;
+    bool miss = false;
+#pragma unroll 1
+    for (int b = 0; b < kPolls; b += kBatch) {
+      if ((int64_t)b * kBlock >= tile) break;
+      uint64_t pv[kBatch];
+      bool have[kBatch];
 #pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    Acc a = (Acc)raw[r][0];
-#pragma unroll
-    for (int j = 1; j < VE; ++j) a += (Acc)raw[r][j];
-    s[r] = a;
-    tsum += a;
-  }
-  // the range's sum goes out before the detailed scan
-  if (CHAINED) {
-    const Acc w = wave_sum(tsum);
-    if (lane == 0) red[wave] = w;
-    __syncthreads();
-    if (tid == 0) {
-      const uint64_t bits = Bits<Acc>::to((red[0] + red[1]) + (red[2] + red[3]));
-      publish(&slots[tile], tag, bits);
-      sums[tile] = bits;
-    }
-  }
-  Acc wexcl[NR];
-#pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    const Acc inc = wave_inclusive_sum(s[r]);
-    wexcl[r] = wave_shift_up1(inc);
-    if (lane == kWave - 1) wtot[r][wave] = inc;
-  }
-  // sum of every earlier range (thread t takes ranges t, t+256, ...): the ones before this
-  // launch's first range are plain words from an earlier call, the others are published by the
-  // workgroups of this launch.  All of a thread's polls are issued together; only the ones not
-  // yet published are repeated.
-  constexpr int kPolls = (CHAINED ? kMaxRanges : kMaxRangesTwo) / kBlock;
-  uint64_t pv[kPolls];
-  bool have[kPolls];
-#pragma unroll
-  for (int i = 0; i < kPolls; ++i) {
-    const int64_t j = tid + (int64_t)i * kBlock;
-    pv[i] = 0ull;
-    have[i] = true;
-    if (j < tile) {
-      if (!CHAINED || j < first_range)
-        pv[i] = sums[j];
-      else
-        have[i] = try_read(&slots[j], tag, &pv[i]);
-    }
-  }
-  if (CHAINED) {
-    bool pending = true;
-    for (int spin = 0; pending && spin < spin_limit; ++spin) {
-      pending = false;
-#pragma unroll
-      for (int i = 0; i < kPolls; ++i) {
-        if (!have[i]) {
-          have[i] = try_read(&slots[tid + (int64_t)i * kBlock], tag, &pv[i]);
-          pending |= !have[i];
+      for (int i = 0; i < kBatch; ++i) {
+        const int64_t j = tid + (int64_t)(b + i) * kBlock;
+        pv[i] = 0ull;
+        have[i] = true;
+        if (j < tile) {
+          if (!CHAINED || j < first_range)
+            pv[i] = sums[j];
+          else
+            have[i] = try_read(&slots[j], tag, &pv[i]);
         }
       }
-      if (pending) __builtin_amdgcn_s_sleep(1);
-    }
-    // Whatever is still missing after the bounded wait is summed here, from the input, with the
-    // tree its own workgroup uses: same bits, and the kernel ends whatever the others do.
+      if (CHAINED) {
+        bool pending = true;
+        for (int spin = 0; pending && spin < spin_limit; ++spin) {
+          pending = false;
 #pragma unroll
-    for (int i = 0; i < kPolls; ++i)
-      if (!have[i]) s_queue[atomicAdd(&s_missing, 1)] = (uint16_t)(tid + i * kBlock);
+          for (int i = 0; i < kBatch; ++i) {
+            if (!have[i]) {
+              have[i] = try_read(&slots[tid + (int64_t)(b + i) * kBlock], tag, &pv[i]);
+              pending |= !have[i];
+            }
+          }
+          if (pending) __builtin_amdgcn_s_sleep(1);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) {
+        const int j = tid + (b + i) * kBlock;
+        if (CHAINED && !have[i]) {
+          atomicOr(&s_missing[j >> 5], 1u << (j & 31));
+          miss = true;
+        } else if (j < tile) {
+          part += Bits<Acc>::from(pv[i]);
+        }
+      }
+    }
+    if (!CHAINED) break;
+    if (!__syncthreads_or(miss)) {
+      failed = false;
+      break;
+    }
+    for (int word = 0; word < kMaxRanges / 32; ++word) {
+      uint32_t bits = s_missing[word];
+      while (bits) {
+        const int j = word * 32 + (__ffs((int)bits) - 1);
+        bits &= bits - 1u;
+        const Acc total = range_total_direct<In, Acc, Out, G>(in, n, j, red);
+        if (tid == 0) publish(&slots[j], tag, Bits<Acc>::to(total));
+      }
+    }
     __syncthreads();
-    const int missing = s_missing;
-    for (int q = 0; q < missing; ++q) {
-      const int j = s_queue[q];
-      const Acc total = range_total<In, Acc, VE, NR>(in, n, j, red);
-#pragma unroll
-      for (int i = 0; i < kPolls; ++i)
-        if (j == tid + i * kBlock) pv[i] = Bits<Acc>::to(total);
-    }
+    if (tid < kMaxRanges / 32) s_missing[tid] = 0u;
+    __syncthreads();
   }
-  Acc part = (Acc)0;
-#pragma unroll
-  for (int i = 0; i < kPolls; ++i)
-    if (tid + (int64_t)i * kBlock < tile) part += Bits<Acc>::from(pv[i]);
   const Acc pw = wave_sum(part);
-  __syncthreads();  // wtot complete; everybody is done reading red
   if (lane == 0) red[wave] = pw;
   __syncthreads();
-  const Acc excl = (red[0] + red[1]) + (red[2] + red[3]);
+  Acc excl = (red[0] + red[1]) + (red[2] + red[3]);
+  // Three passes cannot fail (the second one reads what this workgroup published itself); should
+  // they, the result is marked rather than silently wrong.
+  if (CHAINED && failed) excl = Bits<Acc>::from(0x7ff8dead00000000ull);
+  const Acc wavebase = wave == 0 ? (Acc)0 : wave == 1 ? w0 : wave == 2 ? w0 + w1 : (w0 + w1) + w2;
+  Acc run = (excl + wavebase) + wexcl;
 
-  Acc rowbase = excl;
+  // Results leave through the staging row so that every store instruction of the wave writes
+  // whole 128-byte lines.  Results that fit the caches are stored normally (the search that
+  // follows reads them back); larger ones stream past the caches with non-temporal stores.
+  const bool nt = n * (int64_t)sizeof(Out) > (32ll << 20);
+  constexpr bool kByRun = geo::kOG > G && G * 16 >= 128;  // pieces of G granules of every lane
+  constexpr int kPG = geo::kOG <= G ? geo::kOG : (kByRun ? G : geo::kOG);  // granules per lane and piece
+  constexpr int kPL = (geo::kOG <= G || kByRun) ? kWave : geo::kPiece;   // lanes per piece
+  constexpr int kPieces = (geo::kOG / kPG) * (kWave / kPL);
+  constexpr int kPitch = kPG + 1;
+  static_assert(kPL * kPitch <= geo::kStage, "piece fits the staging row");
+  out_gran o[kPL == kWave ? kPG : geo::kOG];
+  if (kPL != kWave) {
 #pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    Acc acc = rowbase, mine = rowbase;
+    for (int j = 0; j < geo::kOG; ++j)
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      if (w == wave) mine = acc + wexcl[r];
-      acc += wtot[r][w];
+      for (int k = 0; k < geo::kOE; ++k) {
+        run += (Acc)f[j * geo::kOE + k];
+        o[j][k] = (Out)run;
+      }
+  }
+#pragma unroll
+  for (int p = 0; p < kPieces; ++p) {
+    if (kPL == kWave) {
+      // piece p = granules [p*kPG, (p+1)*kPG) of every lane
+#pragma unroll
+      for (int j = 0; j < kPG; ++j) {
+#pragma unroll
+        for (int k = 0; k < geo::kOE; ++k) {
+          run += (Acc)f[(p * kPG + j) * geo::kOE + k];
+          o[j][k] = (Out)run;
+        }
+        stage[lane * kPitch + j] = __builtin_bit_cast(u32x4, o[j]);
+      }
+    } else if (lane / kPL == p) {
+      // piece p = all granules of lanes [p*kPL, (p+1)*kPL)
+      const int l = lane - p * kPL;
+#pragma unroll
+      for (int j = 0; j < geo::kOG; ++j) stage[l * kPitch + j] = __builtin_bit_cast(u32x4, o[j]);
     }
-    rowbase = acc;
-    Acc run = mine;
-    Out o[VE];
+    wave_lds_sync();
+    constexpr int kStores = kPG * kPL / kWave;
+    const bool whole = wbase + geo::kWaveElems <= n;
 #pragma unroll
-    for (int j = 0; j < VE; ++j) {
-      run += (Acc)raw[r][j];
-      o[j] = (Out)run;
+    for (int i = 0; i < kStores; ++i) {
+      const int q = i * kWave + lane;
+      const int l2 = q / kPG, j = q % kPG;
+      const out_gran v = __builtin_bit_cast(out_gran, stage[l2 * kPitch + j]);
+      const int64_t e0 = kPL == kWave
+                             ? wbase + (int64_t)l2 * geo::kEPT + (int64_t)(p * kPG + j) * geo::kOE
+                             : wbase + (int64_t)(p * kPL + l2) * geo::kEPT + (int64_t)j * geo::kOE;
+      if (whole) {
+        store_vec(reinterpret_cast<out_gran *>(out + e0), v, nt);
+      } else {  // ragged end of the input
+#pragma unroll
+        for (int k = 0; k < geo::kOE; ++k)
+          if (e0 + k < n) out[e0 + k] = v[k];
+      }
     }
-    store_slice<Out, VE>(out, base + ((int64_t)r * kBlock + wave * kWave) * VE, n, o, stage[wave],
-                         lane);
+    wave_lds_sync();
   }
 }
 
@@ -512,10 +655,10 @@ enum class Mode { kAuto, kTwoLaunch, kChained };
 // first_changed > 0: the sums of the ranges before the one that holds element first_changed are
 // still in the workspace from the last scan of this array, and `out` still holds the prefix up to
 // there; only the later ranges are summed and scanned again.
-template <typename In, typename Acc, typename Out, int VE, int NR>
+template <typename In, typename Acc, typename Out, int VE, int G>
 int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, bool chained,
                   int64_t first_changed) {
-  const int64_t range_elems = (int64_t)NR * kBlock * VE;
+  const int64_t range_elems = (int64_t)G * kBlock * VE;
   const int64_t ranges = ceil_div64(n, range_elems);
   const int64_t max_ranges = scan_tiles(n, kRows * kBlock * 2);
   uint64_t *sums = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
@@ -523,8 +666,8 @@ int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, b
   const int64_t first = first_changed > 0 ? first_changed / range_elems : 0;
   const dim3 grid((unsigned)(ranges - first)), block(kBlock);
   if (!chained) {
-    range_sum_kernel<In, Acc, VE, NR><<<grid, block, 0, st>>>(in, n, sums, first);
-    scan_ranges_kernel<In, Acc, Out, VE, NR, false><<<grid, block, 0, st>>>(in, out, n, sums, slots,
+    range_sum_kernel<In, Acc, Out, G><<<grid, block, 0, st>>>(in, n, sums, first);
+    scan_ranges_kernel<In, Acc, Out, G, false><<<grid, block, 0, st>>>(in, out, n, sums, slots,
                                                                            first, 0ull, 0);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
@@ -532,7 +675,7 @@ int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, b
   uint64_t tag = g_scan_epoch.fetch_add(1, std::memory_order_relaxed) & kTagMask;
   if (tag == 0) tag = g_scan_epoch.fetch_add(1, std::memory_order_relaxed) & kTagMask;
   const int spin_limit = env_int("GEAR_HIP_SCAN_SPIN_LIMIT", 1 << 14);
-  scan_ranges_kernel<In, Acc, Out, VE, NR, true><<<grid, block, 0, st>>>(in, out, n, sums, slots,
+  scan_ranges_kernel<In, Acc, Out, G, true><<<grid, block, 0, st>>>(in, out, n, sums, slots,
                                                                         first, tag, spin_limit);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -549,12 +692,13 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
   if ((reinterpret_cast<uintptr_t>(in) & (sizeof(In) - 1)) ||
       (reinterpret_cast<uintptr_t>(out) & 15))
     return GEAR_HIP_EALIGN;
-  const int64_t row = (int64_t)kBlock * VE;
-  // GEAR_HIP_SCAN_SINGLE_PASS: 1 = the chained kernel wherever it applies, 0 = never; unset = the
+  // GEAR_HIP_SCAN_SINGLE_PASS: 1 = the chained kernel wherever it applies, 0 = never, 2 = the
+  // ticketed look-back kernel at every size (fp64 sums only; kept for comparisons); unset = the
   // chained kernel for full scans, two launches for the rescan of a suffix.  A launch that is
   // being captured into a graph would replay its tag, so it takes the two launches.
   const int forced = env_int("GEAR_HIP_SCAN_SINGLE_PASS", -1);
-  bool chained = forced < 0 ? first_changed <= 0 : forced != 0;
+  const bool lookback = forced == 2 && std::is_same<Acc, double>::value && first_changed <= 0;
+  bool chained = forced < 0 ? first_changed <= 0 : forced == 1;
   if (chained) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cap) != hipSuccess) {
@@ -563,19 +707,24 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
     }
     if (cap != hipStreamCaptureStatusNone) chained = false;
   }
-  // Ranges of 2, 4 or 8 rows of 256 vectors: the smallest that leave at most 512 ranges, else 8
-  // rows up to 2048 ranges (a workgroup adds up ALL earlier sums, so the chained kernel pays for
-  // the range count squared; 16 rows need 256 registers and run slower than twice 8).  Both
-  // variants cut the input the same way, so a rescan finds the sums of the last full scan.
-  // Beyond 2048 ranges of 8 rows: two launches with up to 8192 ranges of 16 rows.
-  if (ceil_div64(n, 2 * row) <= 512)
+  // Ranges of 2, 4 or 8 granules per thread (2048, 4096 or 8192 fp32 elements): 2 while that
+  // leaves at most 256 ranges, 4 up to 512 ranges, else 8 (a workgroup adds up ALL earlier sums, so
+  // more ranges cost more than they gain once every CU has work).  The chained kernel and the two
+  // launches cut the input the same way, so a rescan finds the sums of the last full scan.
+  // Beyond 4096 ranges the words to poll outweigh the second read: two launches, up to 16384
+  // ranges.  (8-byte elements: ranges of 2 granules would be smaller than the 2048 elements the
+  // workspace is laid out for, so they start at 4.)
+  constexpr int64_t g1 = (int64_t)kBlock * VE;  // elements per range and granule
+  if (lookback) {
+    // fall through to the look-back launch below
+  } else if (VE == 4 && ceil_div64(n, 2 * g1) <= 256)
     return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, chained, first_changed);
-  if (ceil_div64(n, 4 * row) <= 512)
+  else if (ceil_div64(n, 4 * g1) <= 512)
     return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, chained, first_changed);
-  if (ceil_div64(n, 8 * row) <= kMaxRanges)
+  else if (ceil_div64(n, 8 * g1) <= kMaxRanges)
     return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, chained, first_changed);
-  if (ceil_div64(n, 16 * row) <= kMaxRangesTwo)
-    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, false, first_changed);
+  else if (ceil_div64(n, 8 * g1) <= kMaxRangesTwo)
+    return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, false, first_changed);
   // The look-back kernel marks "not published yet" with the word kEmpty, which no fp64 sum of
   // fp32 values can equal but an int64 sum can (-1): int64 scans stop at the two-launch limit.
   if (!std::is_same<Acc, double>::value) return GEAR_HIP_ERANGE;

@@ -177,17 +177,25 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
 
 /* Inclusive prefix sum of fp32 priorities accumulated and written in fp64:
  *     out[i] = sum_{j<=i} (double) in[j]
- * One pass over the input for up to 2048 ranges (n <= 33.5 M): every workgroup publishes the sum
+ * One pass over the input for up to 4096 ranges (n <= 33.5 M): every workgroup publishes the sum
  * of its range and adds the sums of all earlier ranges, with a bounded wait (a workgroup that
- * waited too long sums the missing range itself: same bits, no kernel can hang).  Two launches
- * (range sums, then the scan) beyond that, for a stream under graph capture, and with
+ * waited too long sums the missing range itself and publishes it: same bits, no kernel can
+ * hang).  Two launches (range sums, then the scan) beyond that, for a stream under graph capture,
+ * and with
  * GEAR_HIP_SCAN_SINGLE_PASS=0.  The result is bit-identical in all cases.  Replaces
  * gear::cuda::launch_prefix_sum /
  * one_dimension_prefix_sum (src/cuda/one_dim_prefix_sum.cu:125-273; libgear.core.prefix_sum,
  * :276-278), which is fp32 and only correct for one block.
  * workspace: device memory of at least gear_hip_scan_workspace_bytes(n) bytes, 256-byte aligned;
  * its contents need not be initialised (the call initialises it on `stream`).
- * n may be 0 (nothing is written).  n <= 2^40.  `out` must be 16-byte aligned. */
+ * n may be 0 (nothing is written).  n <= 2^40.  `out` must be 16-byte aligned.
+ * Rounding: inside a range (2048, 4096 or 8192 elements, by n) the prefix is a running sum of a
+ * fixed association; the offset of a range is the separately rounded sum of all earlier ranges.
+ * Both are within 1e-12 (relative) of the sequential fp64 sum, but they are rounded differently,
+ * so across a range boundary out[i+1] can fall below out[i] + in[i+1] by an ulp or two of the
+ * running total; with non-negative input the result is still non-decreasing except where that
+ * difference exceeds in[i+1] (inputs below ~1e-16 of the total).  A search over the prefix treats
+ * such a pair like a run of equal values. */
 size_t gear_hip_scan_workspace_bytes(int64_t n);
 int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspace,
                           size_t workspace_bytes, void *stream);

@@ -22,6 +22,63 @@ def build():
     subprocess.run(["make", "-s", "-B", "-C", _HERE, "liboracle.so"], check=True)
 
 
+REFERENCE_ROOT = "/root/reference"
+_REF = None
+
+
+def build_ref():
+    """Compile the reference's own table-spec sources (src/storage/specs.cc with its headers)
+    behind oracle/ref_specs_glue.cc into oracle/_ref/libref_specs.so.  Needs the reference tree;
+    returns False where it is absent (then a library built earlier is used if it is there)."""
+    if not os.path.isdir(REFERENCE_ROOT):
+        return False
+    subprocess.run(["make", "-s", "-B", "-C", _HERE, "ref"], check=True)
+    return True
+
+
+def ref_specs():
+    """ctypes handle of oracle/_ref/libref_specs.so, or None where it was never built."""
+    global _REF
+    if _REF is None:
+        path = os.path.join(_HERE, "_ref", "libref_specs.so")
+        if not os.path.exists(path):
+            return None
+        _REF = ctypes.CDLL(path)
+        for name in ("ref_sizeof_dtype", "ref_column_size", "ref_table_nbytes", "ref_table_index"):
+            getattr(_REF, name).restype = ctypes.c_int64
+    return _REF
+
+
+def _ref_columns(columns):
+    """columns: [(shape tuple, dtype code)] -> (flat shapes, ndims, dtypes) as ctypes arrays."""
+    flat = [int(d) for shape, _ in columns for d in shape]
+    shapes = (ctypes.c_int64 * max(1, len(flat)))(*flat)
+    ndims = (ctypes.c_int * len(columns))(*[len(shape) for shape, _ in columns])
+    dtypes = (ctypes.c_int * len(columns))(*[int(dt) for _, dt in columns])
+    return shapes, ndims, dtypes
+
+
+def ref_sizeof_dtype(code):
+    return ref_specs().ref_sizeof_dtype(ctypes.c_int(int(code)))
+
+
+def ref_column_size(shape, code):
+    arr = (ctypes.c_int64 * max(1, len(shape)))(*[int(d) for d in shape])
+    return ref_specs().ref_column_size(arr, ctypes.c_int(len(shape)), ctypes.c_int(int(code)))
+
+
+def ref_table_nbytes(trajectory_length, capacity, columns):
+    shapes, ndims, dtypes = _ref_columns(columns)
+    return ref_specs().ref_table_nbytes(ctypes.c_int64(trajectory_length), ctypes.c_int64(capacity),
+                                        ctypes.c_int(len(columns)), shapes, ndims, dtypes)
+
+
+def ref_table_index(columns, name):
+    shapes, ndims, dtypes = _ref_columns(columns)
+    return ref_specs().ref_table_index(ctypes.c_int(len(columns)), shapes, ndims, dtypes,
+                                       name.encode())
+
+
 def lib():
     global _LIB
     if _LIB is None:
