@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per gather launch on config 4, from the two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by a 1 GiB plain copy in the same run) summarised in
 # profiles/subcopy_multi_kernel_config4_hbm_traffic.txt
-MEASURED_GATHER_TRAFFIC_BYTES = 3486579982
+MEASURED_GATHER_TRAFFIC_BYTES = 3486581717
 
 
 def log(msg):
@@ -160,7 +160,17 @@ def run_config4(args):
         ms_pipelined = (time.perf_counter() - t0) * 1e3 / args.steps
 
     payload = B * span * sum(tab.step_bytes)
-    alg_bytes = 2 * payload  # every gathered byte is read once and written once
+    # Every byte of the batch is written once; a window that starts before its trajectory does
+    # (ts < span - 1) reads only the steps that exist, the rest is zero padding.  The read side is
+    # counted from the windows of the timed steps (same seeded draws, sampled again after timing).
+    copied_steps, counted = 0, min(args.steps, 16)
+    for i in range(counted):
+        ops.prefix_sum(dpri, out=prefix)
+        ops.sample_sorted(prefix, u01[args.warmup + i], unit_uniforms=True, sorted_out=flat,
+                          trajectory_length=T, idxs=idxs, tss=tss, lens=lens)
+        copied_steps += int(torch.clamp(tss + 1, max=span).sum().item())
+    read_frac = copied_steps / float(counted * B * span)
+    alg_bytes = payload * (1.0 + read_frac)
     achieved = alg_bytes / (gather_ms * 1e-3) / 1e9
 
     # Yardsticks of the same run: the batch payload moved as ONE contiguous piece, by the library's
@@ -191,8 +201,8 @@ def run_config4(args):
         y64 = ydst[:n8 * 8].view(torch.int64)
         ms_fill = timed_ms(lambda: y64.fill_(1))
         ms_sum = timed_ms(lambda: y64.sum())
-        yard = {"contiguous_copy_slice_kernel_GBps": alg_bytes / (ms_lib * 1e-3) / 1e9,
-                "contiguous_copy_torch_GBps": alg_bytes / (ms_torch * 1e-3) / 1e9,
+        yard = {"contiguous_copy_slice_kernel_GBps": 2 * payload / (ms_lib * 1e-3) / 1e9,
+                "contiguous_copy_torch_GBps": 2 * payload / (ms_torch * 1e-3) / 1e9,
                 "write_only_torch_fill_GBps": n8 * 8 / (ms_fill * 1e-3) / 1e9,
                 "read_only_torch_sum_GBps": n8 * 8 / (ms_sum * 1e-3) / 1e9,
                 "gather_vs_contiguous_copy": ms_lib / gather_ms,
@@ -222,6 +232,8 @@ def run_config4(args):
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                      "avg_launch_ms": gather_ms, "launch_ms_p10_p50_p90": [pct(0.1), pct(0.5), pct(0.9)],
                      "algorithmic_bytes": alg_bytes,
+                     "algorithmic_bytes_if_no_window_were_padded": 2 * payload,
+                     "steps_read_per_step_written": read_frac,
                      "traffic": args.traffic_bytes if args.traffic_bytes is not None else
                      (MEASURED_GATHER_TRAFFIC_BYTES if cap == 1000 else None),
                      "traffic_source": "--traffic-bytes" if args.traffic_bytes is not None else
@@ -783,6 +795,27 @@ def run_scan(args):
     sms = sorted(a.elapsed_time(b) for a, b in ev)
     avg = sum(sms) / len(sms)
     alg = 12 * n
+
+    # Yardsticks of the same run, same n, through torch's own kernels: the plain fp32 -> fp64
+    # conversion copy (the scan's memory pattern without any arithmetic or dependence between
+    # workgroups), an fp64 fill (its writes alone) and torch.cumsum in fp64 (the library scan).
+    def timed_us(fn, reps=50):
+        for _ in range(5):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps * 1e3
+
+    ybuf = torch.empty(n, dtype=torch.float64, device="cuda")
+    yard = {"back_to_back_us": timed_us(lambda: ops.prefix_sum(pri, out=prefix)),
+            "torch_f32_to_f64_copy_us": timed_us(lambda: ybuf.copy_(pri)),
+            "torch_fill_f64_us": timed_us(lambda: ybuf.fill_(1.0)),
+            "torch_cumsum_f64_us": timed_us(lambda: torch.cumsum(pri, 0, dtype=torch.float64, out=ybuf)),
+            "what": "HIP events around 50 back-to-back launches each, same n"}
     variant = {"": "chained single pass (default)", "1": "chained single pass", "0": "two launches",
                "2": "ticketed look-back"}.get(os.environ.get("GEAR_HIP_SCAN_SINGLE_PASS", ""), "?")
     return _line(n / (ms * 1e-3), "priorities/s", args, ms,
@@ -791,7 +824,7 @@ def run_scan(args):
                   "achieved": alg / (avg * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                   "frac": alg / (avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, "avg_launch_ms": avg,
                   "median_launch_ms": sms[len(sms) // 2], "algorithmic_bytes": alg,
-                  "traffic": None})
+                  "traffic": None}, {"yardsticks": yard})
 
 
 def run_topk(args):
@@ -819,6 +852,23 @@ def run_topk(args):
     sms = sorted(a.elapsed_time(b) for a, b in ev)
     avg = sum(sms) / len(sms)
     alg = 4 * n + 12 * k
+
+    def timed_us(fn, reps=50):
+        for _ in range(5):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps * 1e3
+
+    yard = {"back_to_back_us": timed_us(lambda: ops.topk(pri, k, sorted_by_value=by_value)),
+            "torch_topk_us": timed_us(lambda: torch.topk(pri, k, sorted=by_value), reps=10),
+            "torch_sum_read_only_us": timed_us(lambda: pri.sum()),
+            "what": "HIP events around back-to-back launches, same n and k; torch.topk is the "
+                    "library selection, pri.sum() one read of the priorities"}
     return _line(n / (ms * 1e-3), "priorities/s", args, ms,
                  "topk: top %d of %d fp32 priorities, ordered by %s" % (k, n, args.topk_order),
                  {"bound": "hbm", "kernel": "top-k chain (prep, level0, member_hist x2, count, "
@@ -826,7 +876,7 @@ def run_topk(args):
                   "achieved": alg / (avg * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                   "frac": alg / (avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, "avg_launch_ms": avg,
                   "median_launch_ms": sms[len(sms) // 2], "algorithmic_bytes": alg,
-                  "traffic": None})
+                  "traffic": None}, {"yardsticks": yard})
 
 
 def main():

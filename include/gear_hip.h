@@ -194,8 +194,7 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
  * Both are within 1e-12 (relative) of the sequential fp64 sum, but they are rounded differently,
  * so across a range boundary out[i+1] can fall below out[i] + in[i+1] by an ulp or two of the
  * running total; with non-negative input the result is still non-decreasing except where that
- * difference exceeds in[i+1] (inputs below ~1e-16 of the total).  A search over the prefix treats
- * such a pair like a run of equal values. */
+ * difference exceeds in[i+1] (inputs below ~1e-16 of the total). */
 size_t gear_hip_scan_workspace_bytes(int64_t n);
 int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspace,
                           size_t workspace_bytes, void *stream);
