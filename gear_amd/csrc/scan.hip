@@ -296,6 +296,13 @@ template <typename In, typename Out, int G> struct Geo {
 
 // The wave's kWaveElems elements starting at wbase, in blocked order: f[] of lane l holds elements
 // [wbase + l*EPT, wbase + (l+1)*EPT); elements at or beyond n read as 0.
+// Inputs of up to 64 MB are loaded normally: priorities are read again and again (by the next
+// scan, by the top-k before it) and such an array stays in the 256 MB memory-side cache; longer
+// ones stream past the caches with non-temporal loads.
+__host__ __device__ __forceinline__ bool streams_in(int64_t n, size_t elem) {
+  return n * (int64_t)elem > (64ll << 20);
+}
+
 template <typename In, typename Out, int G>
 __device__ __forceinline__ void load_blocked(const In *__restrict__ in, int64_t n, int64_t wbase,
                                              u32x4 *stage, int lane,
@@ -305,10 +312,14 @@ __device__ __forceinline__ void load_blocked(const In *__restrict__ in, int64_t 
   typedef typename Gran<In>::type in_gran;
   if (wbase + geo::kWaveElems <= n) {
     in_vec v[G];
+    const in_vec *src = reinterpret_cast<const in_vec *>(in + wbase + (int64_t)lane * geo::kVE);
+    if (streams_in(n, sizeof(In))) {
 #pragma unroll
-    for (int r = 0; r < G; ++r)
-      v[r] = __builtin_nontemporal_load(
-          reinterpret_cast<const in_vec *>(in + wbase + (int64_t)(r * kWave + lane) * geo::kVE));
+      for (int r = 0; r < G; ++r) v[r] = __builtin_nontemporal_load(src + r * kWave);
+    } else {
+#pragma unroll
+      for (int r = 0; r < G; ++r) v[r] = src[r * kWave];
+    }
 #pragma unroll
     for (int r = 0; r < G; ++r) {
       const int g = r * kWave + lane;
@@ -424,7 +435,8 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
                                                              uint64_t *__restrict__ sums,
                                                              Slot *__restrict__ slots,
                                                              int64_t first_range, uint64_t tag,
-                                                             int spin_limit) {
+                                                             int spin_limit, int stagger,
+                                                             int first_wave) {
   typedef Geo<In, Out, G> geo;
   typedef typename Gran<Out>::type out_gran;
   constexpr int kWaves = kBlock / kWave;
@@ -442,6 +454,17 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
 
   if (CHAINED) {
     if (tid < kMaxRanges / 32) s_missing[tid] = 0u;
+    // All workgroups that fit the GPU at once start within a microsecond.  Left alone, their loads
+    // queue up together and come back in no particular order, every workgroup then waits for the
+    // slowest load of ALL its predecessors, and the whole GPU first reads and then writes.  Starting
+    // workgroup r a little later than r-1 (stagger/1024 clock ticks apiece, the pace at which
+    // memory delivers ranges anyway) makes the ranges arrive in order: early ranges are being
+    // written while late ones are still being read.  The wait is bounded by first_wave * stagger.
+    if (stagger > 0 && blockIdx.x < (unsigned)first_wave) {
+      const unsigned long long until =
+          wall_clock64() + (((unsigned long long)blockIdx.x * (unsigned)stagger) >> 10);
+      while (wall_clock64() < until) __builtin_amdgcn_s_sleep(1);
+    }
   }
   In f[geo::kEPT];
   load_blocked<In, Out, G>(in, n, wbase, stage, lane, f);
@@ -650,7 +673,27 @@ size_t scan_ws_bytes(int64_t n) {
 // every chained launch of the process gets a tag of its own
 std::atomic<uint64_t> g_scan_epoch{1};
 
-enum class Mode { kAuto, kTwoLaunch, kChained };
+// How many workgroups of a kernel the current GPU holds at once, and the rate of wall_clock64().
+struct Residency {
+  int workgroups;
+  int64_t clock_khz;
+};
+Residency residency(const void *kernel) {
+  Residency r{0, 100000};
+  int dev = 0, per_cu = 0, cus = 0, khz = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return r;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kBlock, 0) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return r;
+  }
+  if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) == hipSuccess && khz > 0)
+    r.clock_khz = khz;
+  else
+    (void)hipGetLastError();
+  r.workgroups = per_cu * cus;
+  return r;
+}
 
 // first_changed > 0: the sums of the ranges before the one that holds element first_changed are
 // still in the workspace from the last scan of this array, and `out` still holds the prefix up to
@@ -668,15 +711,24 @@ int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, b
   if (!chained) {
     range_sum_kernel<In, Acc, Out, G><<<grid, block, 0, st>>>(in, n, sums, first);
     scan_ranges_kernel<In, Acc, Out, G, false><<<grid, block, 0, st>>>(in, out, n, sums, slots,
-                                                                           first, 0ull, 0);
+                                                                      first, 0ull, 0, 0, 0);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
   uint64_t tag = g_scan_epoch.fetch_add(1, std::memory_order_relaxed) & kTagMask;
   if (tag == 0) tag = g_scan_epoch.fetch_add(1, std::memory_order_relaxed) & kTagMask;
   const int spin_limit = env_int("GEAR_HIP_SCAN_SPIN_LIMIT", 1 << 14);
-  scan_ranges_kernel<In, Acc, Out, G, true><<<grid, block, 0, st>>>(in, out, n, sums, slots,
-                                                                        first, tag, spin_limit);
+  // Staggered starts pay once several workgroups share a CU (measured: from ~5e6 fp32 elements
+  // on; below that they only delay the launch): 5 ns per range of 8192 fp32 elements.
+  int stagger = 0, first_wave = 0;
+  if (ranges - first > 512) {
+    static const Residency res = residency((const void *)scan_ranges_kernel<In, Acc, Out, G, true>);
+    const int64_t ps = env_int("GEAR_HIP_SCAN_STAGGER_PS", 5000) * (int64_t)(G * 16) / 128;
+    stagger = (int)(ps * res.clock_khz * 1024 / 1000000000ll);
+    first_wave = res.workgroups;
+  }
+  scan_ranges_kernel<In, Acc, Out, G, true><<<grid, block, 0, st>>>(
+      in, out, n, sums, slots, first, tag, spin_limit, stagger, first_wave);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
