@@ -424,6 +424,16 @@ def run_config1(args):
                         tab.traj_stride, tab.step_bytes[c], tab.col_base(c), dst=hd[c])
         n += 1
     cpu_ms = (time.perf_counter() - t0) * 1e3 / n
+    cores = max(1, min(16, os.cpu_count() or 1))
+    t0 = time.perf_counter()
+    nmt = 0
+    while time.perf_counter() - t0 < 2.0:
+        idx = np.sort(rng.integers(0, 4096, size=B))
+        for c in range(4):
+            orc.subcopy(host, idx, np.zeros(B, np.int64), np.full(B, 64, np.int64), False, 0, 64,
+                        tab.traj_stride, tab.step_bytes[c], tab.col_base(c), dst=hd[c], threads=cores)
+        nmt += 1
+    mt_ms = (time.perf_counter() - t0) * 1e3 / nmt
     return _line(B / (ms * 1e-3), "trajectories/s", args, ms,
                  "config1: 4096 x 64 table (obs f32[17], act f32[6], rew f32, done u8), uniform "
                  "batch of 256 full trajectories, sort + 4-column gather",
@@ -433,7 +443,12 @@ def run_config1(args):
                  dict(_graph_extra(B, "trajectories/s", ms_graph),
                       cpu_baseline={"value": B / (cpu_ms * 1e-3), "unit": "trajectories/s",
                                     "cores": 1, "kind": "port", "ms_per_step": cpu_ms,
-                                    "sample": "%d steps of sort + 4-column memset+memcpy gather" % n}))
+                                    "all_cores": {"value": B / (mt_ms * 1e-3),
+                                                  "unit": "trajectories/s", "cores": cores,
+                                                  "ms_per_step": mt_ms, "steps": nmt},
+                                    "cpu_model": cpu_model(),
+                                    "sample": "%d steps of sort + 4-column memset+memcpy gather "
+                                              "(all_cores: windows split over threads)" % n}))
 
 
 def run_config2(args):
@@ -484,6 +499,16 @@ def run_config2(args):
         orc.is_weights(pri, pre[-1], ii, 0.4)
         k += 1
     cpu_ms = (time.perf_counter() - t0) * 1e3 / k
+    cores = max(1, min(16, os.cpu_count() or 1))
+    t0 = time.perf_counter()
+    kmt = 0
+    while time.perf_counter() - t0 < 2.0:
+        uu = rng.random(B, dtype=np.float32)
+        pre = orc.scan_f32_f64(pri, threads=cores)
+        ii = orc.upper_bound_f64(pre, uu, unit_uniforms=True, threads=cores)
+        orc.is_weights(pri, pre[-1], ii, 0.4)
+        kmt += 1
+    mt_ms = (time.perf_counter() - t0) * 1e3 / kmt
     return _line(B / (ms * 1e-3), "draws/s", args, ms,
                  "config2: 1e6 fp32 priorities -> fp64 prefix (one chained single-pass launch), 4096 "
                  "draws, importance weights",
@@ -493,7 +518,11 @@ def run_config2(args):
                  dict(_graph_extra(B, "draws/s", ms_graph),
                       cpu_baseline={"value": B / (cpu_ms * 1e-3), "unit": "draws/s", "cores": 1,
                                     "kind": "port", "ms_per_step": cpu_ms,
-                                    "sample": "%d steps of fp64 scan + 4096 searches + weights" % k}))
+                                    "all_cores": {"value": B / (mt_ms * 1e-3), "unit": "draws/s",
+                                                  "cores": cores, "ms_per_step": mt_ms, "steps": kmt},
+                                    "cpu_model": cpu_model(),
+                                    "sample": "%d steps of fp64 scan + 4096 searches + weights "
+                                              "(all_cores: chunked scan, draws split over threads)" % k}))
 
 
 def run_config3(args):
@@ -572,9 +601,27 @@ def run_config3(args):
                             tab.step_bytes[c], tab.col_base(c), dst=hd[c], want_mask=(c == 0))
             nrun += 1
         cpu_ms = (time.perf_counter() - t0) * 1e3 / nrun
+        cores = max(1, min(16, os.cpu_count() or 1))
+        t0 = time.perf_counter()
+        nmt = 0
+        while nmt < 3 or (time.perf_counter() - t0 < 2.0 and nmt < 2000):
+            pre = orc.scan_i64(hl)
+            traj = orc.sort_i64(orc.upper_bound_i64(pre, crng.random(B), unit_uniforms=True))
+            lens_h = hl[traj]
+            start = (crng.random(B) * (lens_h - (span - 1))).astype(np.int64)
+            for c in range(5):
+                orc.subcopy(host, traj % keep, start, lens_h, False, 0, span, tab.traj_stride,
+                            tab.step_bytes[c], tab.col_base(c), dst=hd[c], want_mask=(c == 0),
+                            threads=cores)
+            nmt += 1
+        mt_ms = (time.perf_counter() - t0) * 1e3 / nmt
         extra["cpu_baseline"] = {
             "value": B / (cpu_ms * 1e-3), "unit": "windows/s", "cores": 1, "kind": "port",
             "ms_per_step": cpu_ms,
+            "all_cores": {"value": B / (mt_ms * 1e-3), "unit": "windows/s", "cores": cores,
+                          "ms_per_step": mt_ms, "steps": nmt,
+                          "what": "windows of the gather split over threads"},
+            "cpu_model": cpu_model(),
             "sample": "%d steps of int64 scan + 1024 searches + sort + 5-column gather with mask, "
                       "table cut to its first %d trajectories" % (nrun, keep)}
     return _line(B / (ms * 1e-3), "windows/s", args, ms,
