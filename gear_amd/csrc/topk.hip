@@ -26,6 +26,8 @@
 // Larger k take the stable LSD radix sort on the inverted key.
 // The streaming loops are sensitive to their instruction count, so they compare floats (one
 // instruction, same order as the keys for non-NaN values) wherever a key is not needed.
+#include <type_traits>
+
 #include "radix_sort.hpp"
 
 namespace gearhip {
@@ -313,6 +315,38 @@ __device__ __forceinline__ void stream_range(const float *__restrict__ p, int64_
   }
 }
 
+// The same for callers that pay for the test of every element against `end`: f(e0, q, whole) with
+// whole = std::true_type when no element of the wave's step lies at or beyond `end`.
+template <typename F>
+__device__ __forceinline__ void stream_range_tagged(const float *__restrict__ p, int64_t begin,
+                                                    int64_t end, int lane, F f) {
+  if (begin >= end) return;
+  float q[kAhead][4];
+#pragma unroll
+  for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
+  for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
+    float qn[kAhead][4];
+    const int64_t s1 = s0 + kAhead * kStep;
+    if (s1 < end) {
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) load_quad(p, s1 + (int64_t)a * kStep + lane * 4, end, qn[a]);
+    }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) {
+      const int64_t w0 = s0 + (int64_t)a * kStep;
+      const int64_t e0 = w0 + lane * 4;
+      if (w0 + kStep <= end)
+        f(e0, q[a], std::true_type{});
+      else if (w0 < end)
+        f(e0, q[a], std::false_type{});
+    }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q[a][j] = qn[a][j];
+  }
+}
+
 // Appends the lane's selected entries (sel[j], in element order) to the wave's list in index
 // order.  `listed` counts every candidate seen, also the ones that no longer fit (wave-uniform).
 __device__ __forceinline__ void list_append(uint64_t *list, int list_cap, int &listed,
@@ -450,11 +484,11 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
   uint64_t *wq = queue[wave];
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
   uint32_t nq = 0;  // candidates of the wave so far (wave-uniform)
-  stream_range(p, begin, end, lane, [&](int64_t e0, const float q[4]) {
+  stream_range_tagged(p, begin, end, lane, [&](int64_t e0, const float q[4], auto whole) {
     uint32_t rem = 0;  // bit j: element j of the lane is a candidate
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const bool valid = e0 + j < end;
+      const bool valid = decltype(whole)::value || e0 + j < end;
       const bool cand = want_lists && valid && q[j] >= lo_f;
       rem |= cand ? 1u << j : 0u;
       // everything else goes to its coarse bin right away
