@@ -11,8 +11,11 @@ from conftest import announce
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
 
+# small sizes, then the sizes at which the range geometry, the staggered start, the streaming
+# loads and the variant change (524 288, 2 097 152, 4 194 304, 16 777 216, 33 554 432, 134 217 728)
 SIZES = [1, 2, 3, 63, 64, 65, 255, 1023, 2047, 2048, 2049, 4095, 4096, 4097, 8191, 8192, 8193,
-         100_000, 1_000_000, 4_194_305, 10_000_003, 34_000_001, 134_300_000]
+         100_000, 524_288, 524_289, 1_000_000, 2_097_153, 4_194_305, 10_000_003, 16_777_217,
+         33_554_433, 34_000_001, 134_300_000]
 
 
 @pytest.fixture(params=["two_launch", "single_pass"])
