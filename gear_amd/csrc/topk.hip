@@ -42,7 +42,11 @@ constexpr int kUniformShift = 18;  // level-0 bins without a sample: the top 14 
 // with a sample: keys below the hint at 12 bits, a middle stretch up to the sample's top in up to
 // kMidBins bins of its own resolution, the rest above
 constexpr int kLowShift = 20, kMidBins = 10240, kMidBinsCoarse = 256;
-constexpr int kSamples = 2048;  // two per thread of one workgroup: more would be bound by the misses one CU can have in flight
+// The sample: 2, 8 or 32 priorities per thread of one workgroup (2048, 8192 or 32768).  One CU
+// sustains about one random miss per 1.2 ns, so the sample is as small as keeps the candidate
+// lists from overflowing: a loose bound lists too much, and after an overflow every later level
+// reads the whole input again.
+constexpr int kMaxSamplesPerThread = 32;
 constexpr uint32_t kNoLists = 0xffffffffu;   // hint_bin: level 0 writes no candidate lists
 constexpr int64_t kBucketMaxK = 131072;      // value order by buckets up to this k
 constexpr int kSortThreads = 1024;           // segment sort workgroup
@@ -377,7 +381,7 @@ __device__ __forceinline__ void list_append(uint64_t *list, int list_cap, int &l
 }
 
 // ---- prep: the sample, the bin map and the zeros ------------------------------------------------------
-// Workgroup 0 looks at kSamples priorities spread over the input (one per stride, at a hashed
+// Workgroup 0 looks at kPer * 1024 priorities spread over the input (one per stride, at a hashed
 // offset inside it) and lays out the level-0 bins around them: the keys below the bin of the
 // `rank`-th largest sample (the hint; bins of the top 14 key bits) are binned coarsely, the
 // stretch from there to the largest sample as finely as kMidBins bins allow, the keys above with
@@ -387,6 +391,7 @@ __device__ __forceinline__ void list_append(uint64_t *list, int list_cap, int &l
 // never correctness.  rank = 0: no sample, uniform bins; every entry is listed when list_all is
 // set (the lists are as long as the waves' ranges), none otherwise.  The other workgroups
 // clear the histograms.
+template <int kPer>  // samples per thread
 __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict__ p, int64_t n,
                                                         uint32_t rank, int list_all, int mid_bins,
                                                         State *state, uint32_t *zero,
@@ -402,10 +407,9 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict_
     }
     return;
   }
-  constexpr int kPer = kSamples / kThreads;
   float v[kPer];
   if (rank != 0u) {
-    const int64_t stride = n / kSamples;  // >= 128 (the caller's condition for a sample), < 2^20
+    const int64_t stride = n / (kPer * kThreads);  // >= 128 (the caller's condition), < 2^20
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const uint32_t s = (uint32_t)(tid + j * kThreads);
@@ -1142,11 +1146,29 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   // would hold most of the input: the levels stream instead).
   const int list_all = g.list_cap >= g.wave_len ? 1 : 0;
   uint32_t rank = 0;
-  if (!list_all && n >= 128 * (int64_t)kSamples && k <= n / 16 &&
+  // Samples per thread: the fewest with which the entries above the hint fit a wave's list with
+  // six standard deviations to spare (a small sample of a long input gives a loose bound: the
+  // rank below cannot go under ~9, whatever the sample's share of k).  No sample at all when even
+  // the largest one would overflow the lists: the levels then stream the input anyway.
+  const auto hint_rank = [&](int per) {
+    const double samples = (double)per * kThreads;
+    const double mu = samples * (double)k / (double)n;
+    return mu + 6.0 * __builtin_sqrt(mu) + 8.0;
+  };
+  const int cap_used = g.list_cap < kQueueCap ? (int)g.list_cap : kQueueCap;
+  const auto lists_hold = [&](int per) {
+    // (the hint is rounded down to a boundary of the coarse bins, up to an eighth of an octave
+    // lower: half as many entries again, and a little, lie above it)
+    const double e = 1.6 * hint_rank(per) / ((double)per * kThreads) * (double)g.wave_len;
+    return e + 6.0 * __builtin_sqrt(e) <= (double)cap_used;
+  };
+  int per = 2;
+  while (per < kMaxSamplesPerThread && !lists_hold(per)) per *= 4;
+  while (per > 2 && n < 128 * (int64_t)per * kThreads) per /= 4;  // strides of 128 elements or more
+  if (!list_all && lists_hold(per) && n >= 128 * (int64_t)per * kThreads && k <= n / 16 &&
       env_int("GEAR_HIP_TOPK_HINT", 1) != 0) {
-    const double mu = (double)kSamples * (double)k / (double)n;
-    const double r = mu + 6.0 * __builtin_sqrt(mu) + 8.0;
-    if (r < kSamples / 4) rank = (uint32_t)r + 1u;
+    const double r = hint_rank(per);
+    if (r < (double)per * kThreads / 4) rank = (uint32_t)r + 1u;
   }
   const int64_t zero_words = (int64_t)((l.zero_end - l.zero_begin) / 4);
   const unsigned zero_blocks = (unsigned)ceil_div64(zero_words, (int64_t)kThreads * 4);
@@ -1154,9 +1176,19 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   // Fine bins pay off in the value-order sort (small, even segments) but cost level 0 an atomic
   // per candidate when its histogram is flushed; the index-ordered selection takes coarse ones.
   const int mid_bins = (sorted_by_value && k <= kBucketMaxK) ? kMidBins : kMidBinsCoarse;
-  prep_kernel<<<dim3(1 + zero_blocks), block, 0, st>>>(
-      priorities, n, rank, list_all, mid_bins, state,
-      reinterpret_cast<uint32_t *>(ws + l.zero_begin), zero_words);
+  {
+    uint32_t *zero = reinterpret_cast<uint32_t *>(ws + l.zero_begin);
+    const dim3 pgrid(1 + zero_blocks);
+    if (per == 2)
+      prep_kernel<2><<<pgrid, block, 0, st>>>(priorities, n, rank, list_all, mid_bins, state, zero,
+                                              zero_words);
+    else if (per == 8)
+      prep_kernel<8><<<pgrid, block, 0, st>>>(priorities, n, rank, list_all, mid_bins, state, zero,
+                                              zero_words);
+    else
+      prep_kernel<32><<<pgrid, block, 0, st>>>(priorities, n, rank, list_all, mid_bins, state,
+                                               zero, zero_words);
+  }
   level0_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len, wave_listed,
                                         lists, (int)g.list_cap);
   // value order by segments: workgroup w of the sort owns the bins that start in the output

@@ -126,6 +126,33 @@ def test_topk_value_order_paths(oracle):
     _check_topk(oracle, ops, wide, 40_000, "priorities over many orders of magnitude, both signs")
 
 
+def _sample_size(n, k):
+    """How many priorities the selection samples: 2, 8 or 32 per thread of one 1024-thread
+    workgroup -- the fewest with which the entries above the hint are expected to fit a wave's
+    candidate list with six standard deviations to spare, with strides of at least 128 elements."""
+    def cdiv(a, b):
+        return -(-a // b)
+
+    wave_len = cdiv(cdiv(n, 4096), 256) * 256            # 256 workgroups of 16 waves, 256-element steps
+    waves = cdiv(n, wave_len * 16) * 16
+    cap = min(max(cdiv(8 * cdiv(k, waves), 64) * 64, 256), 1024, wave_len, 512)
+
+    def rank(per):
+        mu = per * 1024 * k / n
+        return mu + 6.0 * mu ** 0.5 + 8.0
+
+    def lists_hold(per):
+        e = 1.6 * rank(per) / (per * 1024) * wave_len
+        return e + 6.0 * e ** 0.5 <= cap
+
+    per = 2
+    while per < 32 and not lists_hold(per):
+        per *= 4
+    while per > 2 and n < 128 * per * 1024:
+        per //= 4
+    return per * 1024
+
+
 def _sampled_positions(n, samples=2048):
     """Where the selection looks for its sample: one position per stride, at a hashed offset."""
     stride = n // samples
@@ -142,13 +169,14 @@ def test_topk_with_a_misleading_sample(oracle):
     rng = np.random.default_rng(71)
     n = 2_000_000
     base = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
-    pos = _sampled_positions(n)
-    high = base.copy()
-    high[pos] = 1000.0 + rng.random(pos.size, dtype=np.float32)
-    _check_topk(oracle, ops, high, 65_536, "sample overstates (redo)")
-    _check_topk(oracle, ops, high, 1_000, "sample overstates, k below the sampled entries")
+    for k, what in ((65_536, "sample overstates (redo)"),
+                    (1_000, "sample overstates, k below the sampled entries")):
+        pos = _sampled_positions(n, _sample_size(n, k))
+        high = base.copy()
+        high[pos] = 1000.0 + rng.random(pos.size, dtype=np.float32)
+        _check_topk(oracle, ops, high, k, what)
     low = base.copy()
-    low[pos] = 1e-6
+    low[_sampled_positions(n, _sample_size(n, 65_536))] = 1e-6
     _check_topk(oracle, ops, low, 65_536, "sample understates (lists overflow)")
     neg = -base
     _check_topk(oracle, ops, neg, 30_000, "all negative")
