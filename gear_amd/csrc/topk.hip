@@ -838,6 +838,7 @@ constexpr int kLdsEntries = 8192;  // entries per LDS buffer of the segment sort
 constexpr int kStack = 1024;
 
 constexpr int kSortBins = 512;  // 9-bit digits
+constexpr int kNarrowFrom = 2048;  // groups from this size on first look for the bits that differ
 struct SortShared {
   uint32_t cnt[kSortBins + 1];
   uint32_t start[kSortBins + 1];
@@ -846,6 +847,7 @@ struct SortShared {
   uint8_t stk_bits[kStack];   // low bits of the entries still undecided inside the group
   uint8_t stk_flip[kStack];   // the group sits in the second buffer
   int stk_top;
+  uint32_t bits_or_and[4];    // OR (two words) and AND (two words) of a long group's entries
 };
 
 // number of entries of src[lo, hi) larger than `mine`
@@ -859,6 +861,79 @@ __device__ __forceinline__ uint32_t larger_in(const uint64_t *src, uint32_t lo, 
   }
   for (; j < hi; ++j) r += src[j] > mine;
   return r;
+}
+
+// Counting-sort bookkeeping in LDS with the lanes of a wave that share a digit served by ONE
+// atomic: thousands of equal priorities put every entry of a group on the same counter, and LDS
+// atomics on one address are served one lane after the other.  Two rounds peel off the digits
+// of the wave's first unserved lanes when at least eight lanes share them; the rest take plain
+// atomics.  cursor_take returns the old value of cursor[d] for each valid lane (distinct places
+// for the lanes of a digit); count_add only adds.  Called by all lanes of the wave.
+__device__ __forceinline__ uint32_t cursor_take(uint32_t *cursor, uint32_t d, bool valid) {
+  const int lane = (int)(threadIdx.x & 63);
+  const uint64_t lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  uint64_t todo = wave_ballot(valid);
+  uint32_t pos = 0;
+  for (int round = 0; round < 2 && todo != 0ull; ++round) {
+    const int leader = __ffsll((unsigned long long)todo) - 1;
+    const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)d, leader);
+    const uint64_t match = wave_ballot(valid && d == dl) & todo;
+    if (__popcll(match) < 8) break;
+    uint32_t base = 0;
+    if (lane == leader) base = atomicAdd(&cursor[dl], (uint32_t)__popcll(match));
+    base = (uint32_t)__builtin_amdgcn_readlane((int)base, leader);
+    if ((match >> lane) & 1ull) pos = base + (uint32_t)__popcll(match & lt);
+    todo &= ~match;
+  }
+  if ((todo >> lane) & 1ull) pos = atomicAdd(&cursor[d], 1u);
+  return pos;
+}
+__device__ __forceinline__ void count_add(uint32_t *cnt, uint32_t d, bool valid) {
+  const int lane = (int)(threadIdx.x & 63);
+  uint64_t todo = wave_ballot(valid);
+  for (int round = 0; round < 2 && todo != 0ull; ++round) {
+    const int leader = __ffsll((unsigned long long)todo) - 1;
+    const uint32_t dl = (uint32_t)__builtin_amdgcn_readlane((int)d, leader);
+    const uint64_t match = wave_ballot(valid && d == dl) & todo;
+    if (__popcll(match) < 8) break;
+    if (lane == leader) atomicAdd(&cnt[dl], (uint32_t)__popcll(match));
+    todo &= ~match;
+  }
+  if ((todo >> lane) & 1ull) atomicAdd(&cnt[d], 1u);
+}
+
+// A long group often shares most of its remaining bits (thousands of equal priorities: only the
+// index bits differ), and a digit that all entries share would send every one of them to the same
+// LDS counter, one after the other.  Returns how many low bits of src[off, off+len) can still
+// differ (at most rem): the position of the highest bit in which two entries differ, plus one.
+// Called by every thread of the workgroup.
+__device__ __forceinline__ int differing_bits(const uint64_t *src, uint32_t off, uint32_t len,
+                                              int rem, SortShared &sh) {
+  const int tid = threadIdx.x;
+  if (tid < 4) sh.bits_or_and[tid] = tid < 2 ? 0u : 0xffffffffu;
+  __syncthreads();
+  uint64_t o = 0ull, a = ~0ull;
+  for (uint32_t i = tid; i < len; i += kSortThreads) {
+    const uint64_t x = src[off + i];
+    o |= x;
+    a &= x;
+  }
+  for (int d = 32; d >= 1; d >>= 1) {  // the wave's lanes, then one atomic per wave and word
+    o |= (uint64_t)__shfl_xor((unsigned long long)o, d, kWave);
+    a &= (uint64_t)__shfl_xor((unsigned long long)a, d, kWave);
+  }
+  if ((tid & 63) == 0) {
+    atomicOr(&sh.bits_or_and[0], (uint32_t)o);
+    atomicOr(&sh.bits_or_and[1], (uint32_t)(o >> 32));
+    atomicAnd(&sh.bits_or_and[2], (uint32_t)a);
+    atomicAnd(&sh.bits_or_and[3], (uint32_t)(a >> 32));
+  }
+  __syncthreads();
+  uint64_t diff = (((uint64_t)sh.bits_or_and[1] << 32) | sh.bits_or_and[0]) ^
+                  (((uint64_t)sh.bits_or_and[3] << 32) | sh.bits_or_and[2]);
+  __syncthreads();
+  if (rem < 64) diff &= (1ull << rem) - 1ull;
+  return diff ? 64 - __builtin_clzll(diff) : 0;
 }
 
 // Sorts the m entries a[0, m) (descending; only their low `bits` bits can differ) with b as the
@@ -880,7 +955,7 @@ __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t 
     const int top = sh.stk_top;
     if (top == 0) break;
     const uint32_t off = sh.stk_off[top - 1], len = sh.stk_len[top - 1];
-    const int rem = sh.stk_bits[top - 1];
+    int rem = sh.stk_bits[top - 1];
     const bool flip = sh.stk_flip[top - 1] != 0;
     __syncthreads();
     if (tid == 0) sh.stk_top = top - 1;
@@ -893,6 +968,14 @@ __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t 
       }
       __syncthreads();
       continue;
+    }
+    if (len >= (uint32_t)kNarrowFrom) {
+      rem = differing_bits(src, off, len, rem, sh);
+      if (rem == 0) {  // all entries equal: cannot happen (the indices differ), kept for safety
+        for (uint32_t i = tid; i < len; i += kSortThreads) fin[off + i] = src[off + i];
+        __syncthreads();
+        continue;
+      }
     }
     const int nb = rem < 9 ? rem : 9;
     const int shift = rem - nb;
@@ -946,6 +1029,172 @@ __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t 
   }
 }
 
+// The same for a segment that does not fit LDS (thousands of equal or nearly equal priorities
+// among the selected): g0 holds the entries, g1 is the second buffer, both in global memory.
+// Ranking small groups out of global memory would cost a CU one load per pair of entries, so only
+// the counting-sort levels run there: a level cuts its group by 11 bits (ranking a subgroup costs
+// a compare per pair of its members, and all of it is the work of ONE workgroup: short subgroups
+// matter), then runs of whole subgroups that fit LDS are loaded and finished there (small
+// subgroups ranked, longer ones sorted by sort_segment); a subgroup that still exceeds LDS goes
+// down another level.  The level's counters live in the second LDS buffer, which is idle then.
+constexpr int kBigStack = 32;
+constexpr int kBigBits = 11, kBigBins = 1 << kBigBits;
+struct BigShared {
+  uint32_t gstart[kBigBins + 1];
+  uint32_t off[kBigStack], len[kBigStack];
+  uint8_t bits[kBigStack], flip[kBigStack];
+  int top;
+  int nmid;                  // subgroups of the level that fit LDS but are too long to rank
+  uint16_t mid[kBigBins];
+};
+static_assert(kBigBins * 4 <= kLdsEntries * 8, "the counters fit the second LDS buffer");
+static_assert(kBigBins == 2 * kSortThreads, "two counters per thread in the level's scan");
+
+__device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uint32_t m, int bits,
+                                                 uint64_t *__restrict__ fin, SortShared &sh,
+                                                 BigShared &bg, uint64_t *lds_a, uint64_t *lds_b) {
+  const int tid = threadIdx.x;
+  uint32_t *cnt = reinterpret_cast<uint32_t *>(lds_b);
+  constexpr int kInFlight = 4;  // entries a thread has under way in the passes over global memory
+  if (tid == 0) {
+    bg.off[0] = 0u;
+    bg.len[0] = m;
+    bg.bits[0] = (uint8_t)bits;
+    bg.flip[0] = 0;
+    bg.top = 1;
+  }
+  __syncthreads();
+  while (true) {
+    const int top = bg.top;
+    if (top == 0) break;
+    const uint32_t off = bg.off[top - 1], len = bg.len[top - 1];
+    int rem = bg.bits[top - 1];
+    const bool flip = bg.flip[top - 1] != 0;
+    __syncthreads();
+    if (tid == 0) bg.top = top - 1;
+    const uint64_t *src = flip ? g1 : g0;
+    uint64_t *dst = flip ? g0 : g1;
+    rem = differing_bits(src, off, len, rem, sh);
+    if (rem == 0) {
+      for (uint32_t i = tid; i < len; i += kSortThreads) fin[off + i] = src[off + i];
+      __syncthreads();
+      continue;
+    }
+    const int nb = rem < kBigBits ? rem : kBigBits;
+    const int shift = rem - nb;
+    const uint32_t mask = (1u << nb) - 1u;
+    cnt[tid] = 0u;
+    cnt[tid + kSortThreads] = 0u;
+    __syncthreads();
+    for (uint32_t i0 = 0; i0 < len; i0 += kSortThreads * kInFlight) {
+      uint64_t ent[kInFlight];
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const uint32_t i = i0 + (uint32_t)u * kSortThreads + tid;
+        ent[u] = i < len ? src[off + i] : 0ull;
+      }
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const bool valid = i0 + (uint32_t)u * kSortThreads + tid < len;
+        count_add(cnt, mask - (uint32_t)((ent[u] >> shift) & mask), valid);
+      }
+    }
+    __syncthreads();
+    {
+      // exclusive scan of the 2048 counters: thread t owns counters 2t and 2t+1
+      const uint32_t c0 = cnt[2 * tid], c1 = cnt[2 * tid + 1];
+      const int inc = wave_inclusive_sum((int)(c0 + c1));
+      if ((tid & 63) == 63) sh.wsum[tid >> 6] = (uint32_t)inc;
+      __syncthreads();
+      uint32_t before = (uint32_t)inc - (c0 + c1);
+      for (int w = 0; w < (tid >> 6); ++w) before += sh.wsum[w];
+      bg.gstart[2 * tid] = before;
+      bg.gstart[2 * tid + 1] = before + c0;
+      if (tid == kSortThreads - 1) bg.gstart[kBigBins] = before + c0 + c1;
+      if (tid == 0) bg.nmid = 0;
+      __syncthreads();
+      cnt[2 * tid] = before;  // cursors
+      cnt[2 * tid + 1] = before + c0;
+      // subgroups that fit LDS but are too long to rank (one entry of the list per digit at most)
+      if (shift != 0) {
+        if (c0 > (uint32_t)kSmallGroup && c0 <= (uint32_t)kLdsEntries)
+          bg.mid[atomicAdd(&bg.nmid, 1)] = (uint16_t)(2 * tid);
+        if (c1 > (uint32_t)kSmallGroup && c1 <= (uint32_t)kLdsEntries)
+          bg.mid[atomicAdd(&bg.nmid, 1)] = (uint16_t)(2 * tid + 1);
+      }
+      __syncthreads();
+    }
+    for (uint32_t i0 = 0; i0 < len; i0 += kSortThreads * kInFlight) {
+      uint64_t ent[kInFlight];
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const uint32_t i = i0 + (uint32_t)u * kSortThreads + tid;
+        ent[u] = i < len ? src[off + i] : 0ull;
+      }
+#pragma unroll
+      for (int u = 0; u < kInFlight; ++u) {
+        const bool valid = i0 + (uint32_t)u * kSortThreads + tid < len;
+        const uint32_t at = cursor_take(cnt, mask - (uint32_t)((ent[u] >> shift) & mask), valid);
+        if (valid) dst[off + at] = ent[u];
+      }
+    }
+    __syncthreads();
+    // runs of whole subgroups that fit LDS
+    int d0 = 0;
+    while (d0 < kBigBins) {
+      const uint32_t cs = bg.gstart[d0];
+      int d1 = d0;  // the last d with gstart[d] - cs <= kLdsEntries (binary search: gstart ascends)
+      for (int step = kBigBins / 2; step >= 1; step >>= 1)
+        if (d1 + step <= kBigBins && bg.gstart[d1 + step] - cs <= (uint32_t)kLdsEntries) d1 += step;
+      if (d1 + 1 <= kBigBins && bg.gstart[d1 + 1] - cs <= (uint32_t)kLdsEntries) ++d1;
+      if (d1 == d0) {  // subgroup d0 alone exceeds LDS: another level in global memory
+        // (at most m / kLdsEntries such groups exist at a time, far fewer than the stack holds;
+        // with no bits left to cut by, the entries are equal and stay as they are)
+        const int at = bg.top;
+        const bool push = shift != 0 && at < kBigStack;
+        __syncthreads();
+        if (push) {
+          if (tid == 0) {
+            bg.off[at] = off + cs;
+            bg.len[at] = bg.gstart[d0 + 1] - cs;
+            bg.bits[at] = (uint8_t)shift;
+            bg.flip[at] = flip ? 0 : 1;
+            bg.top = at + 1;
+          }
+        } else {
+          const uint32_t ge = bg.gstart[d0 + 1];
+          for (uint32_t i = cs + tid; i < ge; i += kSortThreads) fin[off + i] = dst[off + i];
+        }
+        ++d0;
+        __syncthreads();
+        continue;
+      }
+      const uint32_t ce = bg.gstart[d1], cn = ce - cs;
+      if (cn != 0u) {
+        for (uint32_t i = tid; i < cn; i += kSortThreads) lds_a[i] = dst[off + cs + i];
+        __syncthreads();
+        for (uint32_t i = tid; i < cn; i += kSortThreads) {
+          const uint64_t mine = lds_a[i];
+          const uint32_t d = mask - (uint32_t)((mine >> shift) & mask);
+          const uint32_t gs = bg.gstart[d] - cs, ge = bg.gstart[d + 1] - cs;
+          if (ge - gs <= (uint32_t)kSmallGroup || shift == 0)
+            fin[off + cs + gs + larger_in(lds_a, gs, ge, mine)] = mine;
+        }
+        __syncthreads();
+        // the few subgroups too long to rank (listed when the level was cut) are sorted in place
+        for (int q = 0; q < bg.nmid; ++q) {
+          const int d = bg.mid[q];
+          if (d < d0 || d >= d1) continue;
+          const uint32_t gs = bg.gstart[d] - cs, sz = bg.gstart[d + 1] - bg.gstart[d];
+          sort_segment(lds_a + gs, lds_b, sz, shift, fin + off + cs + gs, sh);
+        }
+        __syncthreads();
+      }
+      d0 = d1;
+    }
+  }
+}
+
 __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
     const float *__restrict__ p, int64_t n, int64_t k, const State *state,
     const uint32_t *__restrict__ hist0, const uint32_t *__restrict__ boff,
@@ -956,6 +1205,7 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
   __shared__ uint64_t lds_a[kLdsEntries], lds_b[kLdsEntries];
   __shared__ uint32_t s_cur;
   __shared__ SortShared sh;
+  __shared__ BigShared bg;
   const int tid = threadIdx.x, lane = tid & 63;
   // The segment ids of the selected entries (a byte each; every workgroup reads them all) do
   // not depend on what this workgroup owns: their loads go out first, sixteen ids per load.
@@ -1075,7 +1325,7 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
   if (in_lds)
     sort_segment(lds_a, lds_b, m, bits, fin + out_lo, sh);
   else
-    sort_segment(buf0 + out_lo, buf1 + out_lo, m, bits, fin + out_lo, sh);
+    sort_big_segment(buf0 + out_lo, buf1 + out_lo, m, bits, fin + out_lo, sh, bg, lds_a, lds_b);
   __syncthreads();
 
   // The segment's stretch of the output, in order.  The value follows from the key (the map is

@@ -126,6 +126,31 @@ def test_topk_value_order_paths(oracle):
     _check_topk(oracle, ops, wide, 40_000, "priorities over many orders of magnitude, both signs")
 
 
+def test_topk_value_order_with_thousands_of_equal_priorities(oracle):
+    """Fresh transitions enter a replay buffer at the maximum priority: thousands of equal
+    priorities above the threshold.  In value order they form one segment that does not fit the
+    sort's LDS buffers (more than 8192 entries): scattered over the array, as one hot stretch of
+    consecutive entries, next to other keys in the same segment, and two such groups."""
+    from gear_amd import ops
+    rng = np.random.default_rng(83)
+    n, k = 3_000_000, 65_536
+    base = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    top = np.float32(base.max())
+    w = base.copy()
+    w[rng.permutation(n)[:30_000]] = top
+    _check_topk(oracle, ops, w, k, "30000 scattered entries at the maximum")
+    w = base.copy()
+    w[1_000_000:1_040_000] = np.float32(10.0)
+    _check_topk(oracle, ops, w, k, "a stretch of 40000 equal entries above the threshold")
+    w = base.copy()
+    w[rng.permutation(n)[:20_000]] = np.float32(10.0)
+    w[2_000_000:2_012_000] = np.float32(10.000001)
+    _check_topk(oracle, ops, w, k, "two long groups of neighbouring keys")
+    w = base.copy()
+    w[rng.permutation(n)[:100_000]] = top
+    _check_topk(oracle, ops, w, 131_072, "100000 entries at the maximum, k = 131072")
+
+
 def _sample_size(n, k):
     """How many priorities the selection samples: 2, 8 or 32 per thread of one 1024-thread
     workgroup -- the fewest with which the entries above the hint are expected to fit a wave's
