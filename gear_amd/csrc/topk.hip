@@ -2,7 +2,7 @@
 //
 // fp32 priorities map to order-preserving uint32 keys, selected top-down in three levels: 16384
 // level-0 bins, then up to 11 and up to 10 bits inside the picked bin.  The launches of one call:
-//   prep      one workgroup draws 2048 samples and lays out the level-0 bins around them (coarse
+//   prep      one workgroup draws 2048 to 32768 samples and lays out the level-0 bins around them (coarse
 //             below the bin that safely lies under the k-th largest priority -- the hint --, fine
 //             from there to the largest sample, the rest above); the others clear the histograms.
 //   level 0   ONE read of the priorities: level-0 histogram (LDS, flushed with atomics) and, per
@@ -22,7 +22,9 @@
 // and puts the entries equal to T straight at the tail of the output; the level-0 histogram says
 // where every bin starts in value order, bins that start in the same stretch of output places
 // form the segment of one workgroup of a last launch, which collects its entries, sorts them
-// (most-significant-digit radix sort in LDS) and writes its stretch of values and indices.
+// (most-significant-digit radix sort in LDS; a segment of more than 8192 entries -- thousands of
+// equal priorities -- is first cut by counting-sort levels in global memory) and writes its
+// stretch of values and indices.
 // Larger k take the stable LSD radix sort on the inverted key.
 // The streaming loops are sensitive to their instruction count, so they compare floats (one
 // instruction, same order as the keys for non-NaN values) wherever a key is not needed.
