@@ -416,3 +416,40 @@ def test_scan_under_graph_capture_replays_correctly(oracle):
         eager = ops.prefix_sum(dp)
         torch.cuda.synchronize()
         assert torch.equal(out, eager), it
+
+
+def test_chained_scans_on_two_streams_next_to_a_busy_gpu():
+    """Workgroups of the chained kernel wait for sums that other workgroups of the same launch
+    publish.  With two such launches in flight on two streams and a third stream keeping every CU
+    busy, late workgroups start when a slot frees: every result must still equal the two-launch
+    result bit for bit (each stream has a workspace of its own)."""
+    from gear_amd import ops
+    rng = np.random.default_rng(17)
+    sizes = [10_000_000, 4_300_000, 1_000_000]
+    pri = [_dev((rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)) for n in sizes]
+    old = os.environ.get("GEAR_HIP_SCAN_SINGLE_PASS")
+    os.environ["GEAR_HIP_SCAN_SINGLE_PASS"] = "0"
+    try:
+        ref = [ops.prefix_sum(p).clone() for p in pri]
+        torch.cuda.synchronize()
+    finally:
+        if old is None:
+            os.environ.pop("GEAR_HIP_SCAN_SINGLE_PASS", None)
+        else:
+            os.environ["GEAR_HIP_SCAN_SINGLE_PASS"] = old
+    s1, s2, s3 = torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.Stream()
+    busy = torch.ones(1 << 27, dtype=torch.float32, device="cuda")
+    outs = [[torch.empty_like(r) for r in ref] for _ in range(2)]
+    announce("chained scans on two streams, 25 rounds")
+    for _ in range(25):
+        with torch.cuda.stream(s3):
+            busy.mul_(1.0001)
+            busy.add_(1.0)
+        for si, st in enumerate((s1, s2)):
+            with torch.cuda.stream(st):
+                for j, p in enumerate(pri):
+                    ops.prefix_sum(p, out=outs[si][j])
+        torch.cuda.synchronize()
+        for si in range(2):
+            for j in range(len(pri)):
+                assert torch.equal(outs[si][j], ref[j])
