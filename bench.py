@@ -6,7 +6,7 @@
 A step is one pass of the hot path over one batch: prefix sum of the per-step priorities, search
 of the batch's seeded uniforms, sort of the drawn indices, split into (trajectory, timestep) and
 the gather of all columns of the windows into contiguous batch tensors.  The default workload is
-BASELINE config 4 (Atari-shape table resident in HBM, 2048 windows of 30 steps).  Rank 0 prints
+benchmark config 4 (Atari-shape table resident in HBM, 2048 windows of 30 steps).  Rank 0 prints
 ONE JSON line; other workloads (--workload) print the same kind of line for that config.
 """
 import argparse
@@ -31,7 +31,7 @@ def log(msg):
 
 
 class AtariTable:
-    """BASELINE config 4 / 5 schema: obs uint8[4,84,84], action int32, reward fp32, done uint8."""
+    """benchmark config 4 / 5 schema: obs uint8[4,84,84], action int32, reward fp32, done uint8."""
     step_bytes = [4 * 84 * 84, 4, 4, 1]
     names = ["obs", "action", "reward", "done"]
 
@@ -935,7 +935,7 @@ def main():
                     help="config 4: trajectories of 1000 steps in the table (1000 = full size)")
     ap.add_argument("--workload", default="config4",
                     choices=["config1", "config2", "config3", "config4", "config5", "scan", "topk"],
-                    help="BASELINE config to run (config4 is the bench line); scan and topk run "
+                    help="benchmark config to run (config4 is the bench line); scan and topk run "
                          "one maintenance kernel chain on its own, for profiles")
     ap.add_argument("--n", type=int, default=10_000_000, help="scan / topk: number of priorities")
     ap.add_argument("--k", type=int, default=65_536, help="topk: entries kept")

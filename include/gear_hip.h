@@ -98,7 +98,7 @@ int gear_hip_host_unregister(void *host_ptr);
  *                pre-zeroes the batch with torch.zeros, gear/loader/offline_loader.py:181-189);
  *                1: the kernel writes the padding zeros itself, so dst may be uninitialised.
  * mask_out       NULL, or uint8[num, span] on the device: 1 where the step holds copied data,
- *                0 where it is padding (no reference counterpart; BASELINE config 3's mask).
+ *                0 where it is padding (no reference counterpart; benchmark config 3's mask).
  * All offsets are 64-bit (the reference's kernel truncates them to int, copy.cu:93-115).
  * Requires n <= dst_stride for every window (GEAR_HIP_EINVAL if span*step_bytes > dst_stride). */
 int gear_hip_subcopy(const void *src, void *dst, int64_t num, const int64_t *idxs,
@@ -156,7 +156,7 @@ int gear_hip_sub(int64_t num, const int64_t *idxs, const int64_t *tss, const int
                  int64_t *dst_offsets, int64_t *copy_lens, void *stream);
 
 /* Sampled flat step index -> window arguments of gear_hip_subcopy, for tables whose priorities
- * are kept per step (BASELINE configs 4 and 5):  f = flat[j] (mod `modulo` when modulo > 0);
+ * are kept per step (benchmark configs 4 and 5):  f = flat[j] (mod `modulo` when modulo > 0);
  *     idxs[j] = f / trajectory_length;  tss[j] = f % trajectory_length;  lens[j] = tss[j] + 1
  * (lens may be NULL).  lens = ts + 1 is the offline convention "timestep == length" of
  * gear/loader/offline_loader.py:200-201,263 applied to a step inside a trajectory: the window
@@ -230,7 +230,7 @@ int gear_hip_scan_f32_f32(const float *in, float *out, int64_t n, void *workspac
 
 /* Same scan over int64 weights (trajectory lengths, include/index/set.h:42), exact in int64
  * (two's complement: weights of either sign, sums wrap like int64 additions).
- * Used for length-weighted trajectory sampling (BASELINE config 3).
+ * Used for length-weighted trajectory sampling (benchmark config 3).
  * n <= 2^26 = 67 108 864, GEAR_HIP_ERANGE beyond (the kernel for longer inputs marks unpublished
  * sums with a word that an int64 sum can equal). */
 int gear_hip_scan_i64(const int64_t *in, int64_t *out, int64_t n, void *workspace,

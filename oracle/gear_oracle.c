@@ -141,7 +141,7 @@ ORACLE_API void oracle_subcopy_mt(const uint8_t *src, uint8_t *dst, int64_t num,
 }
 
 /* ---- A6: prefix sum.  Intent of src/cuda/one_dim_prefix_sum.cu:125-234 (inclusive scan of the
- * priorities), accumulated sequentially in fp64 as BASELINE's "fp64 prefix sum" asks ---------- */
+ * priorities), accumulated sequentially in fp64 as the benchmark's "fp64 prefix sum" asks ---------- */
 ORACLE_API void oracle_scan_f32_f64(const float *in, double *out, int64_t n) {
   double acc = 0.0;
   for (int64_t i = 0; i < n; ++i) {
@@ -258,7 +258,7 @@ ORACLE_API void oracle_upper_bound_i64(const int64_t *prefix, int64_t n, const v
   }
 }
 
-/* Importance weights of BASELINE config 2: w_j = (n * p[idx_j] / total)^(-beta) in fp64,
+/* Importance weights of benchmark config 2: w_j = (n * p[idx_j] / total)^(-beta) in fp64,
  * divided by the maximum over the batch, stored as fp32.  Not in the reference. */
 ORACLE_API void oracle_is_weights(const float *priorities, int64_t n, double total,
                                   const int64_t *idx, int64_t num, double beta, float *out) {

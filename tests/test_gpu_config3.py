@@ -1,4 +1,4 @@
-"""BASELINE config 3 end to end: length-weighted int64 sampler -> length look-up -> start offsets
+"""benchmark config 3 end to end: length-weighted int64 sampler -> length look-up -> start offsets
 -> 5-column window gather with a uint8 attention mask (Decision-Transformer windows).
 
   * full size: 100 000 variable-length trajectories (T = 1000, 104 bytes per step, 10.4 GB in HBM);

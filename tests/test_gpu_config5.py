@@ -1,4 +1,4 @@
-"""BASELINE config 5 as a workload, bit-exact against the CPU oracle for three consecutive steps:
+"""benchmark config 5 as a workload, bit-exact against the CPU oracle for three consecutive steps:
 
     scatter 65 536 new priorities into a 10 000 000-entry array  (src/index/request.cc:41-51)
     -> value-ordered top-65 536                                   (global_sampler.py:195-199)

@@ -35,7 +35,7 @@ def _run_subcopy(ops, schema, table_dev, c, idxs, tss, lens, ofst, span, pad_hea
 
 
 def test_config1_full_trajectories(oracle):
-    """BASELINE config 1 at full size: 4096 x 64 table, 256 uniformly drawn trajectories."""
+    """benchmark config 1 at full size: 4096 x 64 table, 256 uniformly drawn trajectories."""
     from gear_amd import ops
     schema = Schema(CFG1, T=64, capacity=4096)
     table = fill_random(schema, 1001)

@@ -112,7 +112,7 @@ def test_sum_f32(oracle, n):
 
 
 def _boundary_close(prefix, t, idx, rel=1e-9):
-    """Draws within rel * total of a bucket boundary (the exemption BASELINE allows)."""
+    """Draws within rel * total of a bucket boundary (the exemption the benchmark definition allows)."""
     total = prefix[-1]
     lo = np.where(idx > 0, prefix[np.maximum(idx - 1, 0)], 0.0)
     hi = prefix[idx]
@@ -120,7 +120,7 @@ def _boundary_close(prefix, t, idx, rel=1e-9):
 
 
 def test_config2_prioritized_sampling(oracle):
-    """BASELINE config 2 at full size: 1e6 lognormal^0.6 priorities, 4096 fp32 draws in [0, sum),
+    """benchmark config 2 at full size: 1e6 lognormal^0.6 priorities, 4096 fp32 draws in [0, sum),
     indices bit-exact vs the sequential fp64 oracle except boundary-close draws (< 1e-6 of the
     draws), importance weights (N p / sum)^-0.4 / max within 1 ulp of fp32."""
     from gear_amd import ops
@@ -308,7 +308,7 @@ def test_rescan_integer_valued_matches_oracle_exactly(oracle):
 
 def test_split_step_index():
     """flat step index -> (trajectory, timestep, length = timestep + 1), optionally modulo the
-    number of steps in the table (BASELINE config 5 draws from 1e7 priorities over a 2e6-step
+    number of steps in the table (benchmark config 5 draws from 1e7 priorities over a 2e6-step
     table)."""
     from gear_amd import ops
     rng = np.random.default_rng(4)

@@ -59,7 +59,7 @@ def test_column_and_table_sizes_equal_the_reference(ref):
 
 
 def test_baseline_tables_equal_the_reference(ref):
-    """The five BASELINE tables' byte sizes from the reference's TableSpec."""
+    """The five benchmark tables' byte sizes from the reference's TableSpec."""
     atari = [([4, 84, 84], REF_CODE["uint8"]), ([1], REF_CODE["int32"]), ([1], REF_CODE["float32"]),
              ([1], REF_CODE["uint8"])]
     assert ref.ref_table_nbytes(1000, 1000, atari) == 28_233_000_000
