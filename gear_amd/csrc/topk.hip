@@ -202,7 +202,8 @@ Layout layout(int64_t n, int64_t k) {
 // number of entries above every bin at or above the picked one is stored there (where the bin
 // starts in value order), and every non-empty one of those bins is entered into the segment
 // whose stretch of 2^seg_shift output places it starts in (wg_bins: highest bin + 1 and BINS -
-// lowest bin per segment, 0 = none).
+// lowest bin per segment, 0 = none; zeroed by the caller): the workgroups of the launch share
+// that work, every one of them has to call with the same arguments.
 // With no such bin (only possible with NaN priorities, which the float compares of the later
 // levels do not count) the lowest bin is returned and nothing is taken off k_rem.
 struct Pick {
@@ -217,9 +218,14 @@ __device__ __forceinline__ Pick pick_bin(uint32_t k_rem, const uint32_t *hist, u
   __shared__ uint32_t wsum[kWavesPerBlock];
   __shared__ Pick s_pick;
   __shared__ uint32_t s_bin2;  // the bin that holds the rank2-th largest key (rank2 > 0)
-  __shared__ uint32_t s_seg[2 * kMaxBlocks];  // segment table, built in LDS and stored once
+  __shared__ uint32_t s_base[BINS / kWave];  // entries above every 64th bin from the top
   const int tid = threadIdx.x;
-  if (boff && tid < 2 * kMaxBlocks) s_seg[tid] = 0u;
+  // this workgroup's share of the bins whose place in value order is stored (boff): ranks
+  // [r_begin, r_begin + per) from the top; the counts of the first 64 are asked for right away
+  const int per = (((BINS + (int)gridDim.x - 1) / (int)gridDim.x) + kWave - 1) & ~(kWave - 1);
+  const int r_begin = (int)blockIdx.x * per;
+  uint32_t cb0 = 0u;
+  if (boff && tid < kWave && r_begin + tid < BINS) cb0 = hist[BINS - 1 - (r_begin + tid)];
   uint32_t c[kPerThread];  // c[j] = count of bin BINS-1 - tid*kPerThread - j (top down)
   int tsum = 0;
   if (kPerThread % 4 == 0) {
@@ -247,35 +253,66 @@ __device__ __forceinline__ Pick pick_bin(uint32_t k_rem, const uint32_t *hist, u
     s_bin2 = 0u;
   }
   __syncthreads();
-  uint32_t running = (uint32_t)(inc - tsum);
-  for (int w = 0; w < (tid >> 6); ++w) running += wsum[w];
+  // the sums of the waves before this one: one LDS read per lane and a wave sum (a loop over
+  // them would be a chain of dependent LDS reads)
+  const int lane = tid & 63;
+  const uint32_t before =
+      (uint32_t)wave_sum((int)(lane < (tid >> 6) && lane < kWavesPerBlock ? wsum[lane] : 0u));
+  const uint32_t running0 = before + (uint32_t)(inc - tsum);  // entries above the thread's bins
+  const bool active = tid < kActive;
+  // The picked bin is the first one that takes the count up to k_rem: it lies in the ONE thread
+  // whose bins do that, and only that thread walks its bins (16 waves that all walk 16 bins
+  // are bound by instruction issue: 1.5 us).
+  auto find = [&](uint32_t rank, uint32_t *bin_out, uint32_t *rem_out) {
+    if (active && running0 < rank && running0 + (uint32_t)tsum >= rank) {
+      uint32_t r = running0, pb = 0u, pk = 0u;
+      bool found = false;
 #pragma unroll
-  for (int j = 0; j < kPerThread; ++j) {
-    const uint32_t bin = (uint32_t)(BINS - 1 - tid * kPerThread - j);
-    if (tid < kActive && running < k_rem) {
-      // a bin at or above the picked one: everything counted before it is selected
-      if (boff) {
-        boff[bin] = running;
-        if (c[j] != 0u) {  // the segment in whose stretch of the output the bin starts
-          const uint32_t w = running >> seg_shift;
-          atomicMax(&s_seg[2 * w], bin + 1u);
-          atomicMax(&s_seg[2 * w + 1], (uint32_t)BINS - bin);
-        }
+      for (int j = 0; j < kPerThread; ++j) {
+        const bool here = !found && r + c[j] >= rank;
+        pb = here ? (uint32_t)(BINS - 1 - tid * kPerThread - j) : pb;
+        pk = here ? rank - r : pk;
+        found = found || here;
+        r += c[j];
       }
-      if (running + c[j] >= k_rem) {
-        s_pick.bin = bin;
-        s_pick.k_rem = k_rem - running;
-      }
+      *bin_out = pb;
+      if (rem_out) *rem_out = pk;
     }
-    if (rank2 != 0u && tid < kActive && running < rank2 && running + c[j] >= rank2) s_bin2 = bin;
-    running += c[j];
-  }
+  };
+  find(k_rem, &s_pick.bin, &s_pick.k_rem);
+  if (rank2 != 0u) find(rank2, &s_bin2, nullptr);
+  if (boff && (tid * kPerThread) % kWave == 0 && active) s_base[tid * kPerThread / kWave] = running0;
   __syncthreads();
-  if (boff && tid < 2 * kMaxBlocks) wg_bins[tid] = s_seg[tid];
+  // Where the bins at or above the picked one start in value order (the entries above them),
+  // and the segment table.  The workgroups of the launch share the bins, `per` each in runs of
+  // 64: one bin per lane of a wave, after the pick is out, while the other waves go on.  (The
+  // thread that owns 16 bins walking them for this took a microsecond, in workgroup 0 alone
+  // three.)  Bins of one segment are neighbours: the table (zeroed before the launch) hears of
+  // the first and the last non-empty one of a segment in the wave.
+  if (boff) {
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    const uint64_t gt_mask = lane == 63 ? 0ull : (~0ull << (lane + 1));
+    for (int ch = tid >> 6; ch * kWave < per && r_begin + ch * kWave < BINS; ch += kWavesPerBlock) {
+      const int r = r_begin + ch * kWave + lane;  // the bin's rank from the top
+      const uint32_t bin = (uint32_t)(BINS - 1 - r);
+      const uint32_t cnt = ch == 0 ? cb0 : hist[bin];
+      const uint32_t inc_b = (uint32_t)wave_inclusive_sum((int)cnt);
+      const uint32_t above = s_base[(r_begin + ch * kWave) / kWave] + inc_b - cnt;
+      const bool sel = above < k_rem;
+      if (sel) boff[bin] = above;
+      const bool ne = sel && cnt != 0u;
+      const uint32_t w = above >> seg_shift;
+      const uint64_t nem = wave_ballot(ne);
+      const uint64_t lower = nem & lt_mask, upper = nem & gt_mask;
+      const int prev = lower ? 63 - __builtin_clzll(lower) : lane;
+      const int next = upper ? __builtin_ctzll(upper) : lane;
+      const uint32_t w_prev = (uint32_t)__shfl((int)w, prev), w_next = (uint32_t)__shfl((int)w, next);
+      if (ne && (lower == 0ull || w_prev != w)) atomicMax(&wg_bins[2 * w], bin + 1u);
+      if (ne && (upper == 0ull || w_next != w)) atomicMax(&wg_bins[2 * w + 1], (uint32_t)BINS - bin);
+    }
+  }
   if (bin2) *bin2 = s_bin2;
-  const Pick r = s_pick;
-  __syncthreads();  // s_pick and wsum may be written again by a later call
-  return r;
+  return s_pick;  // a kernel calls this once: nothing here is written again
 }
 
 typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -573,14 +610,16 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
   uint32_t lo, hi;  // the keys that are counted
   int shift;        // digit = (key - lo) >> shift
   bool full;
+  // what earlier launches left in the state is asked for before the histogram is walked, not
+  // after it (a round trip to memory each time)
   if (LEVEL == 1) {
-    const Pick r = pick_bin<kBins0>((uint32_t)k, hist_prev, blockIdx.x == 0 ? boff : nullptr,
-                                    wg_bins, seg_shift);
     const BinMap map = state->map;
+    const uint32_t overflow = state->overflow, hint_bin = state->hint_bin;
+    const Pick r = pick_bin<kBins0>((uint32_t)k, hist_prev, boff, wg_bins, seg_shift);
     lo = bin_lo_key(map, r.bin);
     hi = bin_hi_key(map, r.bin);
     shift = level1_shift(bits_of(hi - lo));
-    full = state->overflow != 0u || r.bin < state->hint_bin;
+    full = overflow != 0u || r.bin < hint_bin;
     if (blockIdx.x == 0 && tid == 0) {
       state->prefix[0] = r.bin;
       state->k_rem[0] = r.k_rem;
@@ -589,14 +628,14 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
       state->hi0 = hi;
     }
   } else {
+    const uint32_t lo0 = state->lo0, hi0 = state->hi0, full0 = state->full;
     const Pick r = pick_bin<kBinsR>(state->k_rem[0], hist_prev, nullptr);
-    const uint32_t lo0 = state->lo0, hi0 = state->hi0;
     const int shift1 = level1_shift(bits_of(hi0 - lo0));
     lo = lo0 + (r.bin << shift1);
     hi = lo + ((1u << shift1) - 1u);
     if (hi > hi0 || hi < lo) hi = hi0;
     shift = 0;
-    full = state->full != 0u;
+    full = full0 != 0u;
     if (blockIdx.x == 0 && tid == 0) {
       state->prefix[1] = r.bin;
       state->k_rem[1] = r.k_rem;
@@ -646,14 +685,14 @@ __global__ __launch_bounds__(kThreads) void count_kernel(
   uint64_t *list = lists + gw * list_cap;
   const int m_pre = (int)wave_listed[gw];  // asked for before the pick; used with the lists only
   const uint64_t ent_pre = list[lane];
+  const uint32_t lo0 = state->lo0, hi0 = state->hi0, digit1 = state->prefix[1];
+  const bool full = state->full != 0u;
   const Pick r = pick_bin<kBinsR>(state->k_rem[1], hist2, nullptr);
-  const uint32_t thr =
-      state->lo0 + (state->prefix[1] << level1_shift(bits_of(state->hi0 - state->lo0))) + r.bin;
+  const uint32_t thr = lo0 + (digit1 << level1_shift(bits_of(hi0 - lo0))) + r.bin;
   if (blockIdx.x == 0 && tid == 0) {
     state->prefix[2] = thr;
     state->k_rem[2] = r.k_rem;
   }
-  const bool full = state->full != 0u;
   uint32_t gt = 0, eq = 0;
   if (!full) {
     const int m = m_pre;
