@@ -156,7 +156,7 @@ Geom geom(int64_t n, int64_t k) {
 
 struct Layout {
   size_t hist0, hist1, hist2, wg_bins, boff, wave_listed, wave_ge, block_ge, lists, cidx,
-      cand, cand2, fin, cseg, ckey, skey, sidx, tkey, tidx, shist, zero_begin, zero_end, total;
+      cand, cand2, cseg, ckey, skey, sidx, tkey, tidx, shist, zero_begin, zero_end, total;
 };
 
 Layout layout(int64_t n, int64_t k) {
@@ -168,7 +168,7 @@ Layout layout(int64_t n, int64_t k) {
   l.hist0 = o;  o += kBins0 * sizeof(uint32_t);
   l.hist1 = o;  o += kBinsR * sizeof(uint32_t);
   l.hist2 = o;  o += kBinsR * sizeof(uint32_t);
-  l.wg_bins = o; o += 2 * kMaxBlocks * sizeof(uint32_t);
+  l.wg_bins = o; o += 4 * kMaxBlocks * sizeof(uint32_t);
   l.zero_end = o;
   l.boff = o;   o += kBins0 * sizeof(uint32_t);
   l.wave_listed = o; o += (size_t)kMaxBlocks * kWavesPerBlock * sizeof(uint32_t);
@@ -176,12 +176,11 @@ Layout layout(int64_t n, int64_t k) {
   l.block_ge = o;    o += (size_t)kMaxBlocks * sizeof(uint64_t);
   l.lists = o;  o += align_up((size_t)(g.blocks * kWavesPerBlock * g.list_cap) * 8, 256);
   l.cidx = o;   o += align_up(kk * 4, 256);
-  l.cand = l.cand2 = l.fin = l.cseg = l.ckey = l.skey = l.sidx = l.tkey = l.tidx = l.shist = 0;
+  l.cand = l.cand2 = l.cseg = l.ckey = l.skey = l.sidx = l.tkey = l.tidx = l.shist = 0;
   if (k <= kBucketMaxK) {
     l.ckey = o;  o += align_up(kk * 4, 256);
     l.cand = o;  o += align_up(kk * 8, 256);
     l.cand2 = o; o += align_up(kk * 8, 256);
-    l.fin = o;   o += align_up(kk * 8, 256);
     l.cseg = o;  o += align_up(kk, 256);
   } else {
     const size_t k4 = align_up(kk * 4, 256);
@@ -201,8 +200,9 @@ Layout layout(int64_t n, int64_t k) {
 // and the number of entries still needed inside it to all threads.  When boff is not null the
 // number of entries above every bin at or above the picked one is stored there (where the bin
 // starts in value order), and every non-empty one of those bins is entered into the segment
-// whose stretch of 2^seg_shift output places it starts in (wg_bins: highest bin + 1 and BINS -
-// lowest bin per segment, 0 = none; zeroed by the caller): the workgroups of the launch share
+// whose stretch of 2^seg_shift output places it starts in (wg_bins, four words per segment:
+// highest bin + 1, BINS - lowest bin, ~(entries above the segment), entries above it + its own;
+// 0 = none; zeroed by the caller): the workgroups of the launch share
 // that work, every one of them has to call with the same arguments.
 // With no such bin (only possible with NaN priorities, which the float compares of the later
 // levels do not count) the lowest bin is returned and nothing is taken off k_rem.
@@ -307,8 +307,17 @@ __device__ __forceinline__ Pick pick_bin(uint32_t k_rem, const uint32_t *hist, u
       const int prev = lower ? 63 - __builtin_clzll(lower) : lane;
       const int next = upper ? __builtin_ctzll(upper) : lane;
       const uint32_t w_prev = (uint32_t)__shfl((int)w, prev), w_next = (uint32_t)__shfl((int)w, next);
-      if (ne && (lower == 0ull || w_prev != w)) atomicMax(&wg_bins[2 * w], bin + 1u);
-      if (ne && (upper == 0ull || w_next != w)) atomicMax(&wg_bins[2 * w + 1], (uint32_t)BINS - bin);
+      // highest bin and start of the stretch from the segment's first bin in the wave, lowest
+      // bin and end of the stretch from its last one (the start as its complement: all four are
+      // maxima over the waves that see bins of the segment)
+      if (ne && (lower == 0ull || w_prev != w)) {
+        atomicMax(&wg_bins[4 * w], bin + 1u);
+        atomicMax(&wg_bins[4 * w + 2], ~above);
+      }
+      if (ne && (upper == 0ull || w_next != w)) {
+        atomicMax(&wg_bins[4 * w + 1], (uint32_t)BINS - bin);
+        atomicMax(&wg_bins[4 * w + 3], above + cnt);
+      }
     }
   }
   if (bin2) *bin2 = s_bin2;
@@ -870,7 +879,7 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
 // entries above T inside its key range -- in LDS when they fit, else in its stretch of a
 // global buffer; the places come from a cursor of its own in LDS (global atomics that meet on an
 // address are served one after the other by the memory side) --, sorts them, and writes its
-// stretch of the output.  An entry is key << 32 | ~index, so a larger entry comes earlier in
+// stretch of the output.  An entry is (key - smallest key of the segment's bins) << 32 | ~index, so a larger entry comes earlier in
 // value order (ties: smaller index first) and no two are equal.  The sort is a most-significant-
 // digit radix sort from the highest bit in which the segment's keys can differ: counting sort on
 // 9 bits, groups of up to kSmallGroup entries are ranked directly (every entry counts the larger
@@ -889,6 +898,29 @@ struct SortShared {
   uint8_t stk_flip[kStack];   // the group sits in the second buffer
   int stk_top;
   uint32_t bits_or_and[4];    // OR (two words) and AND (two words) of a long group's entries
+};
+
+// Where a sorted entry goes: place i of the segment's stretch of the output.  The value follows
+// from the key (the map is one to one) except for the two zeros, which share a key: those are
+// read from the input.  (A gather of every value would be bound by the misses one CU can have in
+// flight.)
+struct SegmentOut {
+  const float *p;
+  int64_t n;
+  float *values;
+  int64_t *indices;
+  uint32_t base;
+  uint32_t key_base;  // entries hold key - key_base
+  __device__ __forceinline__ void operator()(uint32_t i, uint64_t ent) const {
+    const uint32_t index = ~(uint32_t)ent, key = (uint32_t)(ent >> 32) + key_base;
+    indices[base + i] = (int64_t)index;
+    if (values)
+      values[base + i] =
+          key != 0x80000000u ? key_to_float(key) : ((int64_t)index < n ? p[index] : 0.0f);
+  }
+  __device__ __forceinline__ SegmentOut shifted(uint32_t by) const {
+    return SegmentOut{p, n, values, indices, base + by, key_base};
+  }
 };
 
 // number of entries of src[lo, hi) larger than `mine`
@@ -978,11 +1010,11 @@ __device__ __forceinline__ int differing_bits(const uint64_t *src, uint32_t off,
 }
 
 // Sorts the m entries a[0, m) (descending; only their low `bits` bits can differ) with b as the
-// second buffer and stores them to fin[0, m); called by every thread of the workgroup.  The two
+// second buffer and hands them to fin(place, entry); called by every thread of the workgroup.  The two
 // callers pass either the LDS buffers or global ones, so that after inlining every access has a
 // known address space.
 __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t m, int bits,
-                                             uint64_t *__restrict__ fin, SortShared &sh) {
+                                             const SegmentOut &fin, SortShared &sh) {
   const int tid = threadIdx.x;
   if (tid == 0) {
     sh.stk_off[0] = 0u;
@@ -1005,7 +1037,7 @@ __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t 
     if (len <= (uint32_t)kSmallGroup || rem == 0) {
       for (uint32_t i = tid; i < len; i += kSortThreads) {
         const uint64_t mine = src[off + i];
-        fin[off + larger_in(src, off, off + len, mine)] = mine;
+        fin(off + larger_in(src, off, off + len, mine), mine);
       }
       __syncthreads();
       continue;
@@ -1013,7 +1045,7 @@ __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t 
     if (len >= (uint32_t)kNarrowFrom) {
       rem = differing_bits(src, off, len, rem, sh);
       if (rem == 0) {  // all entries equal: cannot happen (the indices differ), kept for safety
-        for (uint32_t i = tid; i < len; i += kSortThreads) fin[off + i] = src[off + i];
+        for (uint32_t i = tid; i < len; i += kSortThreads) fin(off + i, src[off + i]);
         __syncthreads();
         continue;
       }
@@ -1055,7 +1087,7 @@ __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t 
       const uint32_t d = mask - (uint32_t)((mine >> shift) & mask);
       const uint32_t gs = sh.start[d], ge = sh.start[d + 1];
       if (ge - gs <= (uint32_t)kSmallGroup || shift == 0) {
-        fin[off + gs + larger_in(dst, off + gs, off + ge, mine)] = mine;
+        fin(off + gs + larger_in(dst, off + gs, off + ge, mine), mine);
       } else if (i == gs) {
         const int at = atomicAdd(&sh.stk_top, 1);
         if (at < kStack) {
@@ -1092,7 +1124,7 @@ static_assert(kBigBins * 4 <= kLdsEntries * 8, "the counters fit the second LDS 
 static_assert(kBigBins == 2 * kSortThreads, "two counters per thread in the level's scan");
 
 __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uint32_t m, int bits,
-                                                 uint64_t *__restrict__ fin, SortShared &sh,
+                                                 const SegmentOut &fin, SortShared &sh,
                                                  BigShared &bg, uint64_t *lds_a, uint64_t *lds_b) {
   const int tid = threadIdx.x;
   uint32_t *cnt = reinterpret_cast<uint32_t *>(lds_b);
@@ -1117,7 +1149,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
     uint64_t *dst = flip ? g0 : g1;
     rem = differing_bits(src, off, len, rem, sh);
     if (rem == 0) {
-      for (uint32_t i = tid; i < len; i += kSortThreads) fin[off + i] = src[off + i];
+      for (uint32_t i = tid; i < len; i += kSortThreads) fin(off + i, src[off + i]);
       __syncthreads();
       continue;
     }
@@ -1204,7 +1236,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
           }
         } else {
           const uint32_t ge = bg.gstart[d0 + 1];
-          for (uint32_t i = cs + tid; i < ge; i += kSortThreads) fin[off + i] = dst[off + i];
+          for (uint32_t i = cs + tid; i < ge; i += kSortThreads) fin(off + i, dst[off + i]);
         }
         ++d0;
         __syncthreads();
@@ -1219,7 +1251,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
           const uint32_t d = mask - (uint32_t)((mine >> shift) & mask);
           const uint32_t gs = bg.gstart[d] - cs, ge = bg.gstart[d + 1] - cs;
           if (ge - gs <= (uint32_t)kSmallGroup || shift == 0)
-            fin[off + cs + gs + larger_in(lds_a, gs, ge, mine)] = mine;
+            fin(off + cs + gs + larger_in(lds_a, gs, ge, mine), mine);
         }
         __syncthreads();
         // the few subgroups too long to rank (listed when the level was cut) are sorted in place
@@ -1227,7 +1259,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
           const int d = bg.mid[q];
           if (d < d0 || d >= d1) continue;
           const uint32_t gs = bg.gstart[d] - cs, sz = bg.gstart[d + 1] - bg.gstart[d];
-          sort_segment(lds_a + gs, lds_b, sz, shift, fin + off + cs + gs, sh);
+          sort_segment(lds_a + gs, lds_b, sz, shift, fin.shifted(off + cs + gs), sh);
         }
         __syncthreads();
       }
@@ -1238,11 +1270,9 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
 
 __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
     const float *__restrict__ p, int64_t n, int64_t k, const State *state,
-    const uint32_t *__restrict__ hist0, const uint32_t *__restrict__ boff,
-    const uint32_t *__restrict__ wg_bins, const uint32_t *__restrict__ ckey,
+    const uint32_t *__restrict__ seg_table, const uint32_t *__restrict__ ckey,
     const uint32_t *__restrict__ cidx, const uint8_t *__restrict__ cseg, uint64_t *buf0,
-    uint64_t *buf1, uint64_t *fin,
-    float *__restrict__ values_out, int64_t *__restrict__ indices_out) {
+    uint64_t *buf1, float *__restrict__ values_out, int64_t *__restrict__ indices_out) {
   __shared__ uint64_t lds_a[kLdsEntries], lds_b[kLdsEntries];
   __shared__ uint32_t s_cur;
   __shared__ SortShared sh;
@@ -1252,7 +1282,8 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
   // not depend on what this workgroup owns: their loads go out first, sixteen ids per load.
   const uint32_t kk = (uint32_t)k;
   const uint32_t pattern = blockIdx.x * 0x01010101u;
-  constexpr int kLoads = 8;
+  constexpr int kLoads = 8;  // covers kBucketMaxK ids
+  static_assert((int64_t)kLoads * kSortThreads * 16 >= kBucketMaxK, "one batch of loads reads every id");
   u32x4 q[kLoads];
 #pragma unroll
   for (int u = 0; u < kLoads; ++u) {
@@ -1260,126 +1291,118 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
     q[u] = u32x4{~pattern, ~pattern, ~pattern, ~pattern};  // no byte matches
     if (i0 + 16 <= kk) q[u] = *reinterpret_cast<const u32x4 *>(cseg + i0);
   }
-  // this workgroup's bins (stored as highest bin + 1 and kBins0 - lowest bin; 0 = none)
-  const uint32_t hi1 = wg_bins[2 * blockIdx.x], loinv = wg_bins[2 * blockIdx.x + 1];
+  // this workgroup's segment: its bins (highest + 1, kBins0 - lowest; 0 = none) and its stretch
+  // of the output, one load; the entries equal to the threshold are not part of any segment
+  const u32x4 mine4 = *reinterpret_cast<const u32x4 *>(seg_table + 4 * blockIdx.x);
+  const uint32_t need_eq = state->k_rem[2];
+  const BinMap map = state->map;
+  if (tid == 0) s_cur = 0u;
+  const uint32_t hi1 = mine4[0], loinv = mine4[1];
   if (hi1 == 0u || loinv == 0u) return;
   const uint32_t hi_bin = hi1 - 1u, lo_bin = (uint32_t)kBins0 - loinv;
-  const uint32_t b0 = state->prefix[0];
-  const uint32_t lo_count = lo_bin == b0 ? state->k_rem[0] - state->k_rem[2] : hist0[lo_bin];
-  const uint32_t out_lo = boff[hi_bin];
-  uint32_t out_hi = boff[lo_bin] + lo_count;
-  if (out_hi > kk) out_hi = kk;  // only out of step with NaN priorities
+  const uint32_t out_lo = ~mine4[2];
+  uint32_t out_hi = mine4[3];
+  if (out_hi > kk - need_eq) out_hi = kk - need_eq;
   if (out_lo >= out_hi) return;
   const uint32_t m = out_hi - out_lo;
   // keys of the segment lie inside the bins' key range
-  const BinMap map = state->map;
   const uint32_t lo_key = bin_lo_key(map, lo_bin);
   const uint32_t hi_key = bin_hi_key(map, hi_bin);
   const bool in_lds = m <= (uint32_t)kLdsEntries;
-  // the positions of the segment's entries are collected first: in LDS (the second buffer,
-  // two per word) or, for a segment that does not fit, in the second global buffer
-  uint32_t *pos_lds = reinterpret_cast<uint32_t *>(lds_b);
-  uint32_t *pos_glb = reinterpret_cast<uint32_t *>(buf1 + out_lo);
-  if (tid == 0) s_cur = 0u;
   __syncthreads();
 
-  // one pass over the segment ids: words without this segment's id are dismissed four ids at a
-  // time; the first kLoads loads per thread are already under way
+  // One pass over the segment ids, then the segment's entries (key, inverted index) are fetched
+  // and kept: in LDS when they fit, else in the segment's stretch of the first global buffer.
+  // All of it is bound by the instructions a CU can issue (1024 threads: 100 instructions per
+  // thread are 0.8 us), so: the ids of a word are compared without branches (exact zero-byte
+  // flags of id ^ own id, gathered into a nibble by a multiplication); the order in which the
+  // entries are collected does not matter (they are sorted next), so a thread counts the hits
+  // of all its loads and the wave takes its places with ONE scan and one LDS atomic; the
+  // fetches of up to four hits per lane are under way together.
   {
-    for (uint32_t r0 = 0; r0 < kk; r0 += kSortThreads * 16 * kLoads) {
-      if (r0 != 0u) {
+    uint64_t hits[kLoads / 4];  // bit 16 * (u % 4) + e: id e of load u is this segment's
 #pragma unroll
-        for (int u = 0; u < kLoads; ++u) {
-          const uint32_t i0 = r0 + ((uint32_t)u * kSortThreads + tid) * 16;
-          q[u] = u32x4{~pattern, ~pattern, ~pattern, ~pattern};
-          if (i0 + 16 <= kk) q[u] = *reinterpret_cast<const u32x4 *>(cseg + i0);
-        }
-      }
+    for (int g = 0; g < kLoads / 4; ++g) {
+      hits[g] = 0ull;
+      if ((uint32_t)g * 4u * kSortThreads * 16u >= kk) continue;  // loads beyond the ids
 #pragma unroll
-      for (int u = 0; u < kLoads; ++u) {
-        const uint32_t i0 = r0 + ((uint32_t)u * kSortThreads + tid) * 16;
-        if (i0 < kk && i0 + 16 > kk) {  // the ragged end of the ids: at most one thread
+      for (int uu = 0; uu < 4; ++uu) {
+        const int u = g * 4 + uu;
+        const uint32_t i0 = ((uint32_t)u * kSortThreads + tid) * 16;
+        if ((kk & 15u) != 0u && i0 < kk && i0 + 16 > kk) {  // the ragged end: at most one thread
           for (int e = 0; e < 16; ++e)
             if (i0 + e < kk)
               q[u][e >> 2] = (q[u][e >> 2] & ~(0xffu << (8 * (e & 3)))) |
                              ((uint32_t)cseg[i0 + e] << (8 * (e & 3)));
         }
-        uint32_t hits = 0;  // bit e: id e of the lane's sixteen is this segment's
+        uint32_t h16 = 0u;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           const uint32_t t = q[u][w] ^ pattern;
-          if (((t - 0x01010101u) & ~t & 0x80808080u) != 0u) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (((t >> (8 * e)) & 0xffu) == 0u) hits |= 1u << (4 * w + e);
-          }
+          // 0x80 in every byte of t that is zero (exact: no borrow between the bytes)
+          const uint32_t z = ~(((t & 0x7f7f7f7fu) + 0x7f7f7f7fu) | t | 0x7f7f7f7fu);
+          // bits 7, 15, 23, 31 -> bits 0..3
+          h16 |= ((((z >> 7) * 0x00204081u) >> 21) & 0xfu) << (4 * w);
         }
-        if (wave_ballot(hits != 0u) == 0ull) continue;
-        const int nc = __popc(hits);
-        const int inc = wave_inclusive_sum(nc);
-        uint32_t base = 0;
-        if (lane == kWave - 1) base = atomicAdd(&s_cur, (uint32_t)inc);
-        base = (uint32_t)__builtin_amdgcn_readlane((int)base, kWave - 1) + (uint32_t)(inc - nc);
-        while (hits) {
-          const int e = __ffs((int)hits) - 1;
-          hits &= hits - 1u;
-          if (base < m) {
-            if (in_lds) pos_lds[base] = i0 + (uint32_t)e; else pos_glb[base] = i0 + (uint32_t)e;
-          }
-          ++base;
-        }
+        hits[g] |= (uint64_t)h16 << (16 * uu);
       }
     }
-  }
-  __syncthreads();
-  // positions -> entries (key, inverted index), many gathers in flight
-  {
-    constexpr int kGathers = 8;
-    for (uint32_t i = tid; i < m; i += kSortThreads * kGathers) {
-      uint32_t pos[kGathers], key[kGathers], idx[kGathers];
+    int nc = 0;
 #pragma unroll
-      for (int u = 0; u < kGathers; ++u) {
-        const uint32_t iu = i + (uint32_t)u * kSortThreads;
-        pos[u] = iu < m ? (in_lds ? pos_lds[iu] : pos_glb[iu]) : kk;
-      }
+    for (int g = 0; g < kLoads / 4; ++g) nc += __popcll(hits[g]);
+    if (wave_ballot(nc != 0) != 0ull) {
+      const int inc = wave_inclusive_sum(nc);
+      uint32_t base = 0;
+      if (lane == kWave - 1) base = atomicAdd(&s_cur, (uint32_t)inc);
+      base = (uint32_t)__builtin_amdgcn_readlane((int)base, kWave - 1) + (uint32_t)(inc - nc);
 #pragma unroll
-      for (int u = 0; u < kGathers; ++u) {
-        key[u] = pos[u] < kk ? ckey[pos[u]] : 0u;
-        idx[u] = pos[u] < kk ? cidx[pos[u]] : 0u;
-      }
+      for (int g = 0; g < kLoads / 4; ++g) {
+        uint64_t h = hits[g];
+        while (wave_ballot(h != 0ull) != 0ull) {
+          constexpr int kFetch = 4;
+          uint32_t pos[kFetch], key[kFetch], idx[kFetch];
 #pragma unroll
-      for (int u = 0; u < kGathers; ++u) {
-        const uint32_t iu = i + (uint32_t)u * kSortThreads;
-        if (iu < m) {
-          const uint64_t ent = ((uint64_t)key[u] << 32) | (uint32_t)~idx[u];
-          if (in_lds) lds_a[iu] = ent; else buf0[out_lo + iu] = ent;
+          for (int f = 0; f < kFetch; ++f) {
+            pos[f] = kk;
+            if (h != 0ull) {
+              const int bit = __builtin_ctzll(h);
+              h &= h - 1ull;
+              pos[f] = ((uint32_t)(g * 4 + (bit >> 4)) * kSortThreads + tid) * 16 + (uint32_t)(bit & 15);
+            }
+          }
+#pragma unroll
+          for (int f = 0; f < kFetch; ++f) {
+            key[f] = pos[f] < kk ? ckey[pos[f]] : 0u;
+            idx[f] = pos[f] < kk ? cidx[pos[f]] : 0u;
+          }
+#pragma unroll
+          for (int f = 0; f < kFetch; ++f) {
+            if (pos[f] < kk) {
+              const uint64_t ent = ((uint64_t)(key[f] - lo_key) << 32) | (uint32_t)~idx[f];
+              if (base < m) {
+                if (in_lds) lds_a[base] = ent; else buf0[out_lo + base] = ent;
+              }
+              ++base;
+            }
+          }
         }
       }
     }
   }
   __syncthreads();
 
-  // bits of the entries that can differ inside the segment: the index, and the key below the
-  // highest bit in which the segment's smallest and largest key differ
-  const uint32_t diff = lo_key ^ hi_key;
-  const int bits = 32 + (diff ? 32 - __builtin_clz(diff) : 0);
+  // An entry holds its key as the distance from the segment's smallest possible key: the bits
+  // in which entries can differ are the index and as many bits as that distance takes for the
+  // largest key, and the digits of the sort cut the key range evenly wherever it lies (the bits
+  // in which the smallest and the largest key themselves differ would be all 24 of them for a
+  // range around a power of two, with every entry in one of two digits).
+  const int bits = 32 + bits_of(hi_key - lo_key);
+  // the sorted entries go straight to the segment's stretch of values and indices
+  const SegmentOut out{p, n, values_out, indices_out, out_lo, lo_key};
   if (in_lds)
-    sort_segment(lds_a, lds_b, m, bits, fin + out_lo, sh);
+    sort_segment(lds_a, lds_b, m, bits, out, sh);
   else
-    sort_big_segment(buf0 + out_lo, buf1 + out_lo, m, bits, fin + out_lo, sh, bg, lds_a, lds_b);
-  __syncthreads();
-
-  // The segment's stretch of the output, in order.  The value follows from the key (the map is
-  // one to one) except for the two zeros, which share a key: those are read from the input.  (A
-  // gather of every value would be bound by the misses one CU can have in flight.)
-  for (uint32_t i = tid; i < m; i += kSortThreads) {
-    const uint64_t ent = fin[out_lo + i];
-    const uint32_t index = ~(uint32_t)ent, key = (uint32_t)(ent >> 32);
-    indices_out[out_lo + i] = (int64_t)index;
-    if (values_out)
-      values_out[out_lo + i] =
-          key != 0x80000000u ? key_to_float(key) : ((int64_t)index < n ? p[index] : 0.0f);
-  }
+    sort_big_segment(buf0 + out_lo, buf1 + out_lo, m, bits, out, sh, bg, lds_a, lds_b);
 }
 static_assert(kSortThreads >= kSortBins, "a thread per digit in the segment sort's scan");
 
@@ -1512,10 +1535,8 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
     uint64_t *cand2 = reinterpret_cast<uint64_t *>(ws + l.cand2);
     uint32_t *bkey = reinterpret_cast<uint32_t *>(ws + l.ckey);
     GEARHIP_WRITE(kBucket, bkey);
-    uint64_t *fin = reinterpret_cast<uint64_t *>(ws + l.fin);
     segment_sort_kernel<<<dim3(kMaxBlocks), dim3(kSortThreads), 0, st>>>(
-        priorities, n, k, state, hist0, boff, wg_bins, bkey, cidx, cseg, cand, cand2, fin,
-        values_out, indices_out);
+        priorities, n, k, state, wg_bins, bkey, cidx, cseg, cand, cand2, values_out, indices_out);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
