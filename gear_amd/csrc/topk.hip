@@ -1309,6 +1309,7 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
   const uint32_t lo_key = bin_lo_key(map, lo_bin);
   const uint32_t hi_key = bin_hi_key(map, hi_bin);
   const bool in_lds = m <= (uint32_t)kLdsEntries;
+  uint32_t *pos_glb = reinterpret_cast<uint32_t *>(buf1 + out_lo);
   __syncthreads();
 
   // One pass over the segment ids, then the segment's entries (key, inverted index) are fetched
@@ -1318,7 +1319,7 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
   // flags of id ^ own id, gathered into a nibble by a multiplication); the order in which the
   // entries are collected does not matter (they are sorted next), so a thread counts the hits
   // of all its loads and the wave takes its places with ONE scan and one LDS atomic; the
-  // fetches of up to four hits per lane are under way together.
+  // fetches of up to eight hits per lane are under way together.
   {
     uint64_t hits[kLoads / 4];  // bit 16 * (u % 4) + e: id e of load u is this segment's
 #pragma unroll
@@ -1355,41 +1356,77 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
       uint32_t base = 0;
       if (lane == kWave - 1) base = atomicAdd(&s_cur, (uint32_t)inc);
       base = (uint32_t)__builtin_amdgcn_readlane((int)base, kWave - 1) + (uint32_t)(inc - nc);
+      if (in_lds) {
 #pragma unroll
-      for (int g = 0; g < kLoads / 4; ++g) {
-        uint64_t h = hits[g];
-        while (wave_ballot(h != 0ull) != 0ull) {
-          constexpr int kFetch = 4;
-          uint32_t pos[kFetch], key[kFetch], idx[kFetch];
+        for (int g = 0; g < kLoads / 4; ++g) {
+          uint64_t h = hits[g];
+          while (wave_ballot(h != 0ull) != 0ull) {
+            constexpr int kFetch = 8;
+            uint32_t pos[kFetch], key[kFetch], idx[kFetch];
 #pragma unroll
-          for (int f = 0; f < kFetch; ++f) {
-            pos[f] = kk;
-            if (h != 0ull) {
-              const int bit = __builtin_ctzll(h);
-              h &= h - 1ull;
-              pos[f] = ((uint32_t)(g * 4 + (bit >> 4)) * kSortThreads + tid) * 16 + (uint32_t)(bit & 15);
-            }
-          }
-#pragma unroll
-          for (int f = 0; f < kFetch; ++f) {
-            key[f] = pos[f] < kk ? ckey[pos[f]] : 0u;
-            idx[f] = pos[f] < kk ? cidx[pos[f]] : 0u;
-          }
-#pragma unroll
-          for (int f = 0; f < kFetch; ++f) {
-            if (pos[f] < kk) {
-              const uint64_t ent = ((uint64_t)(key[f] - lo_key) << 32) | (uint32_t)~idx[f];
-              if (base < m) {
-                if (in_lds) lds_a[base] = ent; else buf0[out_lo + base] = ent;
+            for (int f = 0; f < kFetch; ++f) {
+              pos[f] = kk;
+              if (h != 0ull) {
+                const int bit = __builtin_ctzll(h);
+                h &= h - 1ull;
+                pos[f] = ((uint32_t)(g * 4 + (bit >> 4)) * kSortThreads + tid) * 16 + (uint32_t)(bit & 15);
               }
-              ++base;
             }
+#pragma unroll
+            for (int f = 0; f < kFetch; ++f) {
+              key[f] = pos[f] < kk ? ckey[pos[f]] : 0u;
+              idx[f] = pos[f] < kk ? cidx[pos[f]] : 0u;
+            }
+#pragma unroll
+            for (int f = 0; f < kFetch; ++f) {
+              if (pos[f] < kk) {
+                if (base < m) lds_a[base] = ((uint64_t)(key[f] - lo_key) << 32) | (uint32_t)~idx[f];
+                ++base;
+              }
+            }
+          }
+        }
+      } else {
+        // a long segment (thousands of equal priorities): most ids of a lane are hits, and lanes
+        // that each fetched their own would touch a cache line per lane and load.  The
+        // positions go to the second global buffer first and are fetched in their order.
+#pragma unroll
+        for (int g = 0; g < kLoads / 4; ++g) {
+          uint64_t h = hits[g];
+          while (h != 0ull) {
+            const int bit = __builtin_ctzll(h);
+            h &= h - 1ull;
+            if (base < m)
+              pos_glb[base] = ((uint32_t)(g * 4 + (bit >> 4)) * kSortThreads + tid) * 16 + (uint32_t)(bit & 15);
+            ++base;
           }
         }
       }
     }
   }
   __syncthreads();
+  if (!in_lds) {
+    constexpr int kGathers = 8;
+    for (uint32_t i = tid; i < m; i += kSortThreads * kGathers) {
+      uint32_t pos[kGathers], key[kGathers], idx[kGathers];
+#pragma unroll
+      for (int u = 0; u < kGathers; ++u) {
+        const uint32_t iu = i + (uint32_t)u * kSortThreads;
+        pos[u] = iu < m ? pos_glb[iu] : kk;
+      }
+#pragma unroll
+      for (int u = 0; u < kGathers; ++u) {
+        key[u] = pos[u] < kk ? ckey[pos[u]] : 0u;
+        idx[u] = pos[u] < kk ? cidx[pos[u]] : 0u;
+      }
+#pragma unroll
+      for (int u = 0; u < kGathers; ++u) {
+        const uint32_t iu = i + (uint32_t)u * kSortThreads;
+        if (iu < m) buf0[out_lo + iu] = ((uint64_t)(key[u] - lo_key) << 32) | (uint32_t)~idx[u];
+      }
+    }
+    __syncthreads();
+  }
 
   // An entry holds its key as the distance from the segment's smallest possible key: the bits
   // in which entries can differ are the index and as many bits as that distance takes for the
