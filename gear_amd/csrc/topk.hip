@@ -1065,8 +1065,12 @@ __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t 
       const int inc = wave_inclusive_sum((int)c);
       if ((tid & 63) == 63) sh.wsum[tid >> 6] = (uint32_t)inc;
       __syncthreads();
-      uint32_t before = (uint32_t)inc - c;
-      for (int w = 0; w < (tid >> 6); ++w) before += sh.wsum[w];
+      // sums of the waves before this one: one LDS read per lane and a wave sum, not a chain of
+      // dependent LDS reads
+      const int ln = tid & 63;
+      const uint32_t before =
+          (uint32_t)inc - c +
+          (uint32_t)wave_sum((int)(ln < (tid >> 6) && ln < kSortThreads / kWave ? sh.wsum[ln] : 0u));
       if (tid < kSortBins) {
         sh.start[tid] = before;
         sh.cnt[tid] = before;  // cursors
@@ -1179,8 +1183,10 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
       const int inc = wave_inclusive_sum((int)(c0 + c1));
       if ((tid & 63) == 63) sh.wsum[tid >> 6] = (uint32_t)inc;
       __syncthreads();
-      uint32_t before = (uint32_t)inc - (c0 + c1);
-      for (int w = 0; w < (tid >> 6); ++w) before += sh.wsum[w];
+      const int ln = tid & 63;
+      const uint32_t before =
+          (uint32_t)inc - (c0 + c1) +
+          (uint32_t)wave_sum((int)(ln < (tid >> 6) && ln < kSortThreads / kWave ? sh.wsum[ln] : 0u));
       bg.gstart[2 * tid] = before;
       bg.gstart[2 * tid + 1] = before + c0;
       if (tid == kSortThreads - 1) bg.gstart[kBigBins] = before + c0 + c1;
