@@ -369,13 +369,18 @@ __device__ __forceinline__ void stream_range(const float *__restrict__ p, int64_
 
 // The same for callers that pay for the test of every element against `end`: f(e0, q, whole) with
 // whole = std::true_type when no element of the wave's step lies at or beyond `end`.
-template <typename F>
-__device__ __forceinline__ void stream_range_tagged(const float *__restrict__ p, int64_t begin,
-                                                    int64_t end, int lane, F f) {
-  if (begin >= end) return;
-  float q[kAhead][4];
+// The caller asks for the first kAhead steps itself (stream_first), ahead of work that does
+// not depend on them.
+__device__ __forceinline__ void stream_first(const float *__restrict__ p, int64_t begin, int64_t end,
+                                             int lane, float (&q)[kAhead][4]) {
 #pragma unroll
   for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
+}
+template <typename F>
+__device__ __forceinline__ void stream_range_tagged(const float *__restrict__ p, int64_t begin,
+                                                    int64_t end, int lane, float (&q)[kAhead][4],
+                                                    F f) {
+  if (begin >= end) return;
   for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
     float qn[kAhead][4];
     const int64_t s1 = s0 + kAhead * kStep;
@@ -518,6 +523,12 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
   __shared__ __align__(16) uint32_t h[kBins0];
   __shared__ uint64_t queue[kWavesPerBlock][kQueueCap];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // the first loads of the wave's range go out before the histogram is cleared
+  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t begin = gw * wave_len;
+  const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+  float q0[kAhead][4];
+  stream_first(p, begin, end, lane, q0);
   for (int i = tid; i < kBins0; i += kThreads) h[i] = 0u;
   const uint32_t hint = state->hint_bin;
   const BinMap map = state->map;
@@ -529,14 +540,11 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
   const int low_shift = map.uniform ? kUniformShift : kLowShift;
   const int cap = list_cap < kQueueCap ? list_cap : kQueueCap;
   __syncthreads();
-  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
-  const int64_t begin = gw * wave_len;
-  const int64_t end = begin + wave_len < n ? begin + wave_len : n;
   uint64_t *list = lists + gw * list_cap;
   uint64_t *wq = queue[wave];
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
   uint32_t nq = 0;  // candidates of the wave so far (wave-uniform)
-  stream_range_tagged(p, begin, end, lane, [&](int64_t e0, const float q[4], auto whole) {
+  stream_range_tagged(p, begin, end, lane, q0, [&](int64_t e0, const float q[4], auto whole) {
     uint32_t rem = 0;  // bit j: element j of the lane is a candidate
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
