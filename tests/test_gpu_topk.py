@@ -126,6 +126,26 @@ def test_topk_value_order_paths(oracle):
     _check_topk(oracle, ops, wide, 40_000, "priorities over many orders of magnitude, both signs")
 
 
+def test_topk_value_order_small_inputs_and_narrow_key_ranges(oracle):
+    """The table that says where every bin starts in value order is built by the workgroups of
+    the launch together, however few they are (small inputs), for every k around the numbers of
+    segments; and a segment whose keys lie on both sides of a power of two (where nearly every
+    key bit differs between neighbours) is sorted like any other."""
+    from gear_amd import ops
+    rng = np.random.default_rng(83)
+    ln = lambda n: (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    for n in (300, 5_000, 70_000, 300_000, 1_100_000):
+        w = ln(n)
+        for k in (1, 2, 253, 254, 255, 256, 257, 511, 512, 513, n // 3, n):
+            if k <= min(n, 131_072):
+                _check_topk(oracle, ops, w, k, "n=%d k=%d" % (n, k))
+    around_one = (1.0 + rng.normal(size=2_000_000) * 1e-4).astype(np.float32)
+    _check_topk(oracle, ops, around_one, 65_536, "priorities around 1.0")
+    _check_topk(oracle, ops, around_one, 1_000_000, "priorities around 1.0, half of them")
+    around_zero = (rng.normal(size=1_000_000) * 1e-30).astype(np.float32)
+    _check_topk(oracle, ops, around_zero, 100_000, "priorities around 0, both signs")
+
+
 def test_topk_value_order_with_thousands_of_equal_priorities(oracle):
     """Fresh transitions enter a replay buffer at the maximum priority: thousands of equal
     priorities above the threshold.  In value order they form one segment that does not fit the
