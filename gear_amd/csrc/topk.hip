@@ -504,6 +504,10 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict_
   }
 }
 
+// Adds 1 to cnt[d] for every valid lane; lanes of the wave that share a counter take one atomic
+// (defined with the segment sort).  Called by all lanes of the wave.
+__device__ __forceinline__ void count_add(uint32_t *cnt, uint32_t d, bool valid);
+
 // ---- level 0: ONE read of the priorities --------------------------------------------------------------
 // Every entry is counted in its level-0 bin (LDS histogram, flushed with atomics); the
 // candidates -- entries at or above the hint, about one in fifty -- are also listed per wave, in
@@ -556,17 +560,23 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
     }
     uint64_t with;  // lanes that still hold a candidate; a lane rarely has two: one round
     while ((with = wave_ballot(rem != 0u)) != 0ull) {
+      bool over = false;
+      uint32_t over_bin = 0u;
       if (rem != 0u) {
         const int j = __ffs((int)rem) - 1;
         rem &= rem - 1u;
         const float x = j == 0 ? q[0] : (j == 1 ? q[1] : (j == 2 ? q[2] : q[3]));
         const uint32_t at = nq + (uint32_t)__popcll(with & lt_mask);
-        if (at < (uint32_t)cap)
+        if (at < (uint32_t)cap) {
           wq[at] = ((uint64_t)__float_as_uint(x) << 32) | (uint32_t)(e0 + j);
-        else
-          atomicAdd(&h[bin_of(map, order_key(x))], 1u);
+        } else {
+          over = true;
+          over_bin = bin_of(map, order_key(x));
+        }
       }
       nq += (uint32_t)__popcll(with);
+      // the queue is full (the lists are given up): masses of equal priorities share a bin
+      if (nq > (uint32_t)cap) count_add(h, over_bin, over);
     }
   });
   if (want_lists) {
@@ -677,10 +687,11 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
     stream_range(p, begin, end, lane, [&](int64_t e0, const float q[4]) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (e0 + j < end && q[j] >= lo_f && q[j] <= hi_f) {
-          const uint32_t key = order_key(q[j]);
-          if (key >= lo && key <= hi) atomicAdd(&h[(key - lo) >> shift], 1u);
-        }
+        const bool near = e0 + j < end && q[j] >= lo_f && q[j] <= hi_f;
+        if (wave_ballot(near) == 0ull) continue;
+        // masses of equal priorities share a digit: one atomic per wave then
+        const uint32_t key = order_key(q[j]);
+        count_add(h, (key - lo) >> shift, near && key >= lo && key <= hi);
       }
     });
   }
@@ -803,12 +814,15 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
 
   // pos = the entry's place in index order among the selected, e = its rank among the entries
   // equal to T.
-  auto emit = [&](bool selected, bool is_eq, uint32_t pos, uint32_t e, uint32_t index, uint32_t key) {
+  // `have` says that `value` is the entry's priority (the streaming path has it at hand; from a
+  // list it is read from the input: the key does not tell the two zeros apart).
+  auto emit = [&](bool selected, bool is_eq, uint32_t pos, uint32_t e, uint32_t index, uint32_t key,
+                  auto have, float value) {
     selected = selected && pos < (uint32_t)k;  // out of step only with NaN priorities
     if (FLAVOUR == kDirect) {
       if (selected) {
         indices_out[pos] = (int64_t)index;
-        if (values_out) values_out[pos] = p[index];
+        if (values_out) values_out[pos] = decltype(have)::value ? value : p[index];
       }
     } else if (FLAVOUR == kPairs) {
       if (selected) {
@@ -820,7 +834,7 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
       // bucket sort skips them (it takes keys above T only)
       if (selected && is_eq && ties_at + e < (uint32_t)k) {
         indices_out[ties_at + e] = (int64_t)index;
-        if (values_out) values_out[ties_at + e] = p[index];
+        if (values_out) values_out[ties_at + e] = decltype(have)::value ? value : p[index];
       }
       if (selected) {
         ckey[pos] = key;
@@ -843,7 +857,8 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
       const uint32_t g = gt_run + (uint32_t)__popcll(bg & lt_mask);
       const uint32_t e = eq_run + (uint32_t)__popcll(be & lt_mask);
       const bool selected = is_gt || (is_eq && e < need_eq);
-      emit(selected, is_eq, g + (e < need_eq ? e : need_eq), e, (uint32_t)ent, key);
+      emit(selected, is_eq, g + (e < need_eq ? e : need_eq), e, (uint32_t)ent, key,
+           std::false_type{}, 0.0f);
       gt_run += (uint32_t)__popcll(bg);
       eq_run += (uint32_t)__popcll(be);
     }
@@ -859,6 +874,8 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
     for (int j = 0; j < 4; ++j)
       if (e0 + j < end) s += q[j] > thr_f ? (1 << 16) : (q[j] == thr_f ? 1 : 0);
     if (wave_ballot(s != 0) == 0ull) return;
+    // nothing of the step is selected once the ties needed are placed and no entry is above T
+    if (eq_run >= need_eq && wave_ballot((s >> 16) != 0) == 0ull) return;
     const int inc = wave_inclusive_sum(s);
     const int total = wave_read_lane(inc, kWave - 1);
     const int before = inc - s;
@@ -870,7 +887,7 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
       const bool is_gt = valid && q[j] > thr_f, is_eq = valid && q[j] == thr_f;
       const bool selected = is_gt || (is_eq && e < need_eq);
       emit(selected, is_eq, g + (e < need_eq ? e : need_eq), e, (uint32_t)(e0 + j),
-           is_gt ? order_key(q[j]) : thr);
+           is_gt ? order_key(q[j]) : thr, std::true_type{}, q[j]);
       g += is_gt;
       e += is_eq;
     }
