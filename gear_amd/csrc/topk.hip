@@ -548,6 +548,26 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
   uint64_t *wq = queue[wave];
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
   uint32_t nq = 0;  // candidates of the wave so far (wave-uniform)
+  // Lists that hold whole ranges with no hint (short inputs): every element is a candidate and
+  // its place in the wave's list is its place in the wave's range -- nothing to queue or order.
+  const bool whole_ranges = want_lists && hint == 0u && (int64_t)list_cap >= wave_len;
+  if (whole_ranges) {
+    stream_range_tagged(p, begin, end, lane, q0, [&](int64_t e0, const float q[4], auto whole) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (decltype(whole)::value || e0 + j < end) {
+          const uint32_t key = order_key(q[j]);
+          atomicAdd(&h[bin_of(map, key)], 1u);
+          list[e0 + j - begin] = ((uint64_t)key << 32) | (uint32_t)(e0 + j);
+        }
+      }
+    });
+    if (lane == 0) wave_listed[gw] = begin < end ? (uint32_t)(end - begin) : 0u;
+    __syncthreads();
+    for (int i = tid; i < kBins0; i += kThreads)
+      if (h[i]) atomicAdd(&hist0[i], h[i]);
+    return;
+  }
   stream_range_tagged(p, begin, end, lane, q0, [&](int64_t e0, const float q[4], auto whole) {
     uint32_t rem = 0;  // bit j: element j of the lane is a candidate
 #pragma unroll
