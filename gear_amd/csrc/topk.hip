@@ -516,6 +516,7 @@ __device__ __forceinline__ void count_add(uint32_t *cnt, uint32_t d, bool valid)
 // or two candidates, so whatever is done per candidate there is paid per step); after the
 // stream the wave orders its queue by index, bins the candidates and writes the list, all lanes
 // busy.  A candidate that finds the queue full is binned at once and the lists are given up.
+constexpr uint32_t kRankAll = 160;  // queues up to this length are ordered by comparing every pair
 constexpr int kQueueCap = 512;  // candidates per wave held in LDS; longer lists overflow
 
 __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restrict__ p, int64_t n,
@@ -607,15 +608,34 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
       const uint64_t mine = wq[i];
       const uint32_t index = (uint32_t)mine;
       uint32_t r = 0;
-      const uint32_t m8 = m & ~7u;
-      for (uint32_t j = 0; j < m8; j += 8) {  // eight LDS reads in flight
-        uint32_t x[8];
+      if (m <= kRankAll) {
+        const uint32_t m8 = m & ~7u;
+        for (uint32_t j = 0; j < m8; j += 8) {  // eight LDS reads in flight
+          uint32_t x[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) x[u] = (uint32_t)wq[j + u];
+          for (int u = 0; u < 8; ++u) x[u] = (uint32_t)wq[j + u];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) r += x[u] < index;
+          for (int u = 0; u < 8; ++u) r += x[u] < index;
+        }
+        for (uint32_t j = m8; j < m; ++j) r += (uint32_t)wq[j] < index;
+      } else {
+        // A long queue: it holds the steps of the stream one after the other, and only inside
+        // a step the order of arrival (every lane's first candidate, then the second ones) is
+        // not the order of the indices: the entry looks at its neighbours of the same step.
+        const uint32_t first = (uint32_t)begin;  // a multiple of kStep
+        const uint32_t step = (index - first) / (uint32_t)kStep;
+        r = i;
+        for (uint32_t j = i; j-- > 0u;) {
+          const uint32_t other = (uint32_t)wq[j];
+          if ((other - first) / (uint32_t)kStep != step) break;
+          r -= other > index;
+        }
+        for (uint32_t j = i + 1; j < m; ++j) {
+          const uint32_t other = (uint32_t)wq[j];
+          if ((other - first) / (uint32_t)kStep != step) break;
+          r += other < index;
+        }
       }
-      for (uint32_t j = m8; j < m; ++j) r += (uint32_t)wq[j] < index;
       const uint32_t key = order_key(__uint_as_float((uint32_t)(mine >> 32)));
       atomicAdd(&h[bin_of(map, key)], 1u);
       list[r] = ((uint64_t)key << 32) | index;
