@@ -122,6 +122,8 @@ def test_topk_value_order_paths(oracle):
     _check_topk(oracle, ops, ln(262_144), 1_000, "smallest input with a sample")
     _check_topk(oracle, ops, ln(262_143), 1_000, "largest input without a sample")
     _check_topk(oracle, ops, ln(30_000_000), 65_536, "long input")
+    # ~220 candidates per wave: the queues are ordered by the same-step neighbours
+    _check_topk(oracle, ops, ln(60_000_000), 65_536, "longer input, long candidate queues")
     wide = (rng.normal(size=1_000_000) * np.exp(rng.normal(size=1_000_000) * 8)).astype(np.float32)
     _check_topk(oracle, ops, wide, 40_000, "priorities over many orders of magnitude, both signs")
 
