@@ -44,6 +44,13 @@ constexpr int kUniformShift = 18;  // level-0 bins without a sample: the top 14 
 // with a sample: keys below the hint at 12 bits, a middle stretch up to the sample's top in up to
 // kMidBins bins of its own resolution, the rest above
 constexpr int kLowShift = 20, kMidBins = 10240, kMidBinsCoarse = 256;
+// Keys of one level-0 bin differ in at most this many low bits, whichever stretch it lies in:
+// level 1 resolves the top 11 of them, level 2 the rest.
+constexpr int kMaxBinBits = 21;
+static_assert(kLowShift <= kMaxBinBits && kUniformShift <= kMaxBinBits, "coarse bins within the levels' reach");
+static_assert((1ll << (32 - kMaxBinBits)) <= kMidBins, "the middle stretch can always be cut finely enough");
+static_assert((1ll << 32 >> kLowShift) + kMidBins + (1ll << (32 - kMaxBinBits)) <= kBins0,
+              "the stretch above the largest sample keeps enough bins for bins of 2^kMaxBinBits keys");
 // The sample: 2, 8 or 32 priorities per thread of one workgroup (2048, 8192 or 32768).  One CU
 // sustains about one random miss per 1.2 ns, so the sample is as small as keeps the candidate
 // lists from overflowing: a loose bound lists too much, and after an overflow every later level
@@ -491,7 +498,11 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict_
     map.a_end = (hint14 << kUniformShift) & ~((1u << kLowShift) - 1u);
     map.b_last = ((top14 + 1u) << kUniformShift) - 1u;  // wraps to the last key for the top bin
     const uint32_t span = map.b_last - map.a_end;
-    while ((span >> map.b_shift) >= (uint32_t)mid_bins) ++map.b_shift;
+    // (a bin never spans more than 2^kMaxBinBits keys -- the two levels below resolve 11 bits
+    // each --: a middle stretch too wide for mid_bins bins of that size gets more of them, at most
+    // 2048, which the budget of kMidBins covers)
+    while (map.b_shift < (uint32_t)kMaxBinBits && (span >> map.b_shift) >= (uint32_t)mid_bins)
+      ++map.b_shift;
     map.nb0 = map.a_end >> kLowShift;
     map.nc0 = map.nb0 + (span >> map.b_shift) + 1u;
     const uint32_t rest = 0xffffffffu - map.b_last;  // keys above the middle stretch

@@ -126,6 +126,14 @@ def test_topk_value_order_paths(oracle):
     _check_topk(oracle, ops, ln(60_000_000), 65_536, "longer input, long candidate queues")
     wide = (rng.normal(size=1_000_000) * np.exp(rng.normal(size=1_000_000) * 8)).astype(np.float32)
     _check_topk(oracle, ops, wide, 40_000, "priorities over many orders of magnitude, both signs")
+    # candidates from 1e-38 to 100: the stretch of keys between the hint and the largest sample
+    # is more than a quarter of all keys, and no level-0 bin may be wider than the two levels
+    # below it can resolve (the index-ordered selection asks for few, wide bins there)
+    tiny = (rng.random(10_000_000) * 1e-38).astype(np.float32)
+    tiny[9_000_000:9_014_000] += np.float32(100.0)
+    _check_topk(oracle, ops, tiny, 59_000, "denormals and a stretch of 100.0")
+    tiny[rng.permutation(10_000_000)[:30_000]] = rng.random(30_000, dtype=np.float32) * 1e30
+    _check_topk(oracle, ops, tiny, 59_000, "denormals up to 1e30")
 
 
 def test_topk_value_order_small_inputs_and_narrow_key_ranges(oracle):
