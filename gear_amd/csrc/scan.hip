@@ -4,7 +4,7 @@
 // granules of its range, adds them up in order, and one DPP wave scan per range joins the
 // threads (a wave-private LDS row turns the row-major order of the memory instructions, 1 KiB of
 // consecutive addresses per wave and instruction, into that blocked order and back):
-//  * chained single pass, up to 4096 ranges: scan_ranges_kernel<CHAINED = true>.  A workgroup
+//  * chained single pass, up to 4096 ranges: scan_ranges_kernel<kChained>.  A workgroup
 //    keeps its range in registers, publishes the range's sum and adds the sums of ALL earlier
 //    ranges (fixed order: bit-reproducible), then writes the prefix: the input is read once.
 //    Range r belongs to workgroup r (no ticket).  A published sum travels as three 64-bit words
@@ -15,14 +15,21 @@
 //    predecessor's range itself, with the same reduction tree, and publishes it on the
 //    predecessor's behalf, so no kernel can spin forever and the result does not change.
 //  * two launches, up to 16384 ranges (n <= 134 M fp32): range_sum_kernel writes the sum of every
-//    range; scan_ranges_kernel<CHAINED = false> re-reads its range (now in L2 / MALL), adds the
+//    range; scan_ranges_kernel<kTwoLaunches> re-reads its range (now in L2 / MALL), adds the
 //    sums of all earlier ranges and writes the prefix.  No workgroup waits for another one.  Used
 //    for long inputs, under stream capture (a captured launch would replay its tag) and for the
 //    incremental rescan of a suffix.
-//  * beyond that: scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone,
-//    incl[t] = sum of tiles 0..t; wave 0 looks back 64 predecessors at a time, ballots pick the
-//    nearest published inclusive value; tile numbers come from an atomic ticket).
+//  * beyond that: three launches -- range_sum_kernel, range_prefix_kernel (ONE workgroup scans the
+//    range sums in a fixed order) and scan_ranges_kernel<kPrefixed>, which finds the sum of all
+//    earlier ranges in one word.  Same bits on every run, and for the rescan of a suffix.
+//  * scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone, incl[t] = sum of
+//    tiles 0..t; wave 0 looks back 64 predecessors at a time, ballots pick the nearest published
+//    inclusive value; tile numbers come from an atomic ticket), runs only when asked for
+//    (GEAR_HIP_SCAN_SINGLE_PASS=2, for comparisons): what it adds up depends on which
+//    predecessors had published what, so two runs can differ in the last bit.
 #include <atomic>
+#include <chrono>
+#include <random>
 #include <type_traits>
 
 #include "wave.hpp"
@@ -424,12 +431,44 @@ __global__ __launch_bounds__(kBlock) void range_sum_kernel(const In *__restrict_
   if (threadIdx.x == 0) sums[range] = Bits<Acc>::to(total);
 }
 
+// Exclusive prefix of the range sums by ONE workgroup, in an order that depends on nothing but
+// the number of ranges (thread t adds its stretch of the sums one after the other, the stretches'
+// totals are scanned, the stretch is walked again): the third launch between the two above for
+// inputs of more ranges than a workgroup can add up by itself.
+constexpr int kPrefixThreads = 1024;
+template <typename Acc>
+__global__ __launch_bounds__(kPrefixThreads) void range_prefix_kernel(
+    const uint64_t *__restrict__ sums, uint64_t *__restrict__ prefix, int64_t ranges) {
+  __shared__ Acc wtot[kPrefixThreads / kWave];
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  const int64_t per = ceil_div64(ranges, kPrefixThreads);
+  const int64_t lo = (int64_t)tid * per, hi = lo + per < ranges ? lo + per : ranges;
+  Acc mine = (Acc)0;
+  for (int64_t i = lo; i < hi; ++i) mine += Bits<Acc>::from(sums[i]);
+  const Acc inc = wave_inclusive_sum(mine);
+  if (lane == kWave - 1) wtot[wave] = inc;
+  __syncthreads();
+  Acc run = (Acc)0;
+  for (int w = 0; w < wave; ++w) run += wtot[w];
+  run += wave_shift_up1(inc);
+  for (int64_t i = lo; i < hi; ++i) {
+    prefix[i] = Bits<Acc>::to(run);
+    run += Bits<Acc>::from(sums[i]);
+  }
+}
+
 // sums[r]   plain range sums (kept between calls: the incremental rescan reuses the ones before
 //           its first range)
-// slots[r]  CHAINED only: the same sums as tagged words, for the workgroups of this launch
-// spin_limit  CHAINED only: polls of a missing predecessor before the workgroup sums that range
+// slots[r]  chained: the same sums as tagged words, for the workgroups of this launch; prefixed:
+//           8-byte words, the sum of all ranges before r
+// spin_limit  chained only: polls of a missing predecessor before the workgroup sums that range
 //           itself
-template <typename In, typename Acc, typename Out, int G, bool CHAINED>
+enum RangeMode {
+  kTwoLaunches = 0,  // every workgroup adds up the sums of the ranges before its own
+  kChained = 1,      // ... and the sums of this launch's ranges arrive while it runs
+  kPrefixed = 2      // the sum of all earlier ranges is ready: slots holds one word per range
+};
+template <typename In, typename Acc, typename Out, int G, int MODE>
 __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restrict__ in,
                                                              Out *__restrict__ out, int64_t n,
                                                              uint64_t *__restrict__ sums,
@@ -439,8 +478,9 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
                                                              int first_wave) {
   typedef Geo<In, Out, G> geo;
   typedef typename Gran<Out>::type out_gran;
+  constexpr bool CHAINED = MODE == kChained;
   constexpr int kWaves = kBlock / kWave;
-  constexpr int kPolls = (CHAINED ? kMaxRanges : kMaxRangesTwo) / kBlock;
+  constexpr int kPolls = MODE == kPrefixed ? 0 : (CHAINED ? kMaxRanges : kMaxRangesTwo) / kBlock;
   constexpr int kBatch = 4;
   __shared__ u32x4 stage_all[kWaves][geo::kStage];
   __shared__ Acc wtot[kWaves];
@@ -555,6 +595,7 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
   if (lane == 0) red[wave] = pw;
   __syncthreads();
   Acc excl = (red[0] + red[1]) + (red[2] + red[3]);
+  if (MODE == kPrefixed) excl = Bits<Acc>::from(reinterpret_cast<const uint64_t *>(slots)[tile]);
   // Three passes cannot fail (the second one reads what this workgroup published itself); should
   // they, the result is marked rather than silently wrong.
   if (CHAINED && failed) excl = Bits<Acc>::from(0x7ff8dead00000000ull);
@@ -670,8 +711,29 @@ size_t scan_ws_bytes(int64_t n) {
   return kHeaderBytes + align_up((size_t)tiles * (8 + sizeof(Slot)), 256);
 }
 
-// every chained launch of the process gets a tag of its own
-std::atomic<uint64_t> g_scan_epoch{1};
+// Every chained launch of the process gets a tag of its own, and one that nothing else is likely
+// to have left in memory: a workspace need not be initialised, and what it holds is rarely
+// random -- small integers (indices, counts, sums of them) are common, and so would be the tags
+// 1, 2, 3 ... of an earlier process whose memory this one was given.  The launch counter
+// therefore starts at a random place and goes through a bijection of the 42-bit tags that
+// scatters neighbouring counts (multiplications by odd numbers and xor-shifts).
+std::atomic<uint64_t> g_scan_epoch{0};
+uint64_t next_tag() {
+  static const uint64_t seed = [] {
+    std::random_device rd;
+    uint64_t s = ((uint64_t)rd() << 32) ^ (uint64_t)rd();
+    s ^= (uint64_t)std::chrono::steady_clock::now().time_since_epoch().count();
+    return s;
+  }();
+  for (;;) {
+    uint64_t x = (g_scan_epoch.fetch_add(1, std::memory_order_relaxed) + seed) & kTagMask;
+    x = (x * 0x2545F4914F5ull) & kTagMask;
+    x ^= x >> 21;
+    x = (x * 0x1B03738712Full) & kTagMask;
+    x ^= x >> 19;
+    if (x != 0ull && x != kTagMask) return x;  // all-zero and all-one words are common too
+  }
+}
 
 // How many workgroups of a kernel the current GPU holds at once, and the rate of wall_clock64().
 struct Residency {
@@ -710,24 +772,32 @@ int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, b
   const dim3 grid((unsigned)(ranges - first)), block(kBlock);
   if (!chained) {
     range_sum_kernel<In, Acc, Out, G><<<grid, block, 0, st>>>(in, n, sums, first);
-    scan_ranges_kernel<In, Acc, Out, G, false><<<grid, block, 0, st>>>(in, out, n, sums, slots,
-                                                                      first, 0ull, 0, 0, 0);
+    if (ranges <= kMaxRangesTwo) {
+      scan_ranges_kernel<In, Acc, Out, G, kTwoLaunches><<<grid, block, 0, st>>>(
+          in, out, n, sums, slots, first, 0ull, 0, 0, 0);
+    } else {
+      // more ranges than a workgroup adds up by itself: their prefix comes from a launch in
+      // between (into the words that the chained variant uses for its slots)
+      range_prefix_kernel<Acc><<<dim3(1), dim3(kPrefixThreads), 0, st>>>(
+          sums, reinterpret_cast<uint64_t *>(slots), ranges);
+      scan_ranges_kernel<In, Acc, Out, G, kPrefixed><<<grid, block, 0, st>>>(
+          in, out, n, sums, slots, first, 0ull, 0, 0, 0);
+    }
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
-  uint64_t tag = g_scan_epoch.fetch_add(1, std::memory_order_relaxed) & kTagMask;
-  if (tag == 0) tag = g_scan_epoch.fetch_add(1, std::memory_order_relaxed) & kTagMask;
+  const uint64_t tag = next_tag();
   const int spin_limit = env_int("GEAR_HIP_SCAN_SPIN_LIMIT", 1 << 14);
   // Staggered starts pay once several workgroups share a CU (measured: from ~5e6 fp32 elements
   // on; below that they only delay the launch): 5 ns per range of 8192 fp32 elements.
   int stagger = 0, first_wave = 0;
   if (ranges - first > 512) {
-    static const Residency res = residency((const void *)scan_ranges_kernel<In, Acc, Out, G, true>);
+    static const Residency res = residency((const void *)scan_ranges_kernel<In, Acc, Out, G, kChained>);
     const int64_t ps = env_int("GEAR_HIP_SCAN_STAGGER_PS", 5000) * (int64_t)(G * 16) / 128;
     stagger = (int)(ps * res.clock_khz * 1024 / 1000000000ll);
     first_wave = res.workgroups;
   }
-  scan_ranges_kernel<In, Acc, Out, G, true><<<grid, block, 0, st>>>(
+  scan_ranges_kernel<In, Acc, Out, G, kChained><<<grid, block, 0, st>>>(
       in, out, n, sums, slots, first, tag, spin_limit, stagger, first_wave);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
@@ -775,11 +845,12 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
     return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, chained, first_changed);
   else if (ceil_div64(n, 8 * g1) <= kMaxRanges)
     return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, chained, first_changed);
-  else if (ceil_div64(n, 8 * g1) <= kMaxRangesTwo)
+  else
     return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, false, first_changed);
-  // The look-back kernel marks "not published yet" with the word kEmpty, which no fp64 sum of
-  // fp32 values can equal but an int64 sum can (-1): int64 scans stop at the two-launch limit.
-  if (!std::is_same<Acc, double>::value) return GEAR_HIP_ERANGE;
+  // (The look-back kernel marks "not published yet" with the word kEmpty, which no fp64 sum of
+  // fp32 values can equal but an int64 sum can (-1): fp64 sums only.  Its sums depend on which
+  // predecessors had published what when a workgroup looked: two runs can differ in the last
+  // bit, which is why it is not used unless asked for.)
   const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
   uint32_t *ticket = static_cast<uint32_t *>(ws);
   uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);

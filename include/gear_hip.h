@@ -181,8 +181,8 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
  * of its range and adds the sums of all earlier ranges, with a bounded wait (a workgroup that
  * waited too long sums the missing range itself and publishes it: same bits, no kernel can
  * hang).  Two launches (range sums, then the scan) beyond that, for a stream under graph capture,
- * and with
- * GEAR_HIP_SCAN_SINGLE_PASS=0.  The result is bit-identical in all cases.  Replaces
+ * and with GEAR_HIP_SCAN_SINGLE_PASS=0; three (a launch in between scans the range sums) beyond
+ * 16384 ranges (n > 134 M).  The result is bit-identical in all cases and on every run.  Replaces
  * gear::cuda::launch_prefix_sum /
  * one_dimension_prefix_sum (src/cuda/one_dim_prefix_sum.cu:125-273; libgear.core.prefix_sum,
  * :276-278), which is fp32 and only correct for one block.
@@ -218,7 +218,7 @@ int gear_hip_scan_f32_f64_static(const float *in, double *out, int64_t n, void *
  * with the same n, and since then only in[first_changed .. n) changed.  Then out[i] is
  * recomputed from the start of the range that holds first_changed onwards, reusing the range sums
  * kept in the workspace; the result is bit-identical to a full gear_hip_scan_f32_f64.
- * first_changed >= n: nothing to do; first_changed = 0 or n > 134 M: a full scan. */
+ * first_changed >= n: nothing to do; first_changed = 0: a full scan. */
 int gear_hip_rescan_f32_f64(const float *in, double *out, int64_t n, int64_t first_changed,
                             void *workspace, size_t workspace_bytes, void *stream);
 
@@ -231,8 +231,7 @@ int gear_hip_scan_f32_f32(const float *in, float *out, int64_t n, void *workspac
 /* Same scan over int64 weights (trajectory lengths, include/index/set.h:42), exact in int64
  * (two's complement: weights of either sign, sums wrap like int64 additions).
  * Used for length-weighted trajectory sampling (benchmark config 3).
- * n <= 2^26 = 67 108 864, GEAR_HIP_ERANGE beyond (the kernel for longer inputs marks unpublished
- * sums with a word that an int64 sum can equal). */
+ * n <= 2^40. */
 int gear_hip_scan_i64(const int64_t *in, int64_t *out, int64_t n, void *workspace,
                       size_t workspace_bytes, void *stream);
 

@@ -343,16 +343,80 @@ def test_scan_i64_signed_weights_with_range_sums_of_minus_one(oracle, n, scan_va
         assert np.array_equal(got, oracle.scan_i64(v))
 
 
-def test_scan_i64_beyond_its_limit_is_refused():
+def test_scans_of_more_ranges_than_a_workgroup_adds_up():
+    """Beyond 16384 ranges (134 M fp32 / 67 M int64 elements) a launch in between scans the range
+    sums: same bits on every run and for the rescan of a suffix, exact on integers, int64 sums of
+    -1 included."""
+    from gear_amd import ops
+    n = (1 << 27) + 5001
+    g = torch.Generator(device="cuda").manual_seed(11)
+    announce("scan f32->f64 n=%d (three launches)" % n)
+    w = torch.randint(0, 1000, (n,), device="cuda", generator=g).float()
+    got = ops.prefix_sum(w).clone()
+    assert torch.equal(got, torch.cumsum(w.double(), 0))          # integers: exact in any order
+    w = torch.rand(n, device="cuda", generator=g)
+    first = ops.prefix_sum(w).clone()
+    again = ops.prefix_sum(w).clone()
+    assert torch.equal(first, again)
+    ref = torch.cumsum(w.double(), 0)
+    assert float((first - ref).abs().max() / ref[-1]) <= 1e-12
+    del ref, again
+    state = ops.PrefixState()
+    state.scan(w)
+    for k in (1, 8191, 50_000_000, n - 1):
+        w[k:] = torch.rand(n - k, device="cuda", generator=g)
+        announce("rescan n=%d from %d (three launches)" % (n, k))
+        got = state.scan(w, first_changed=k)
+        full = ops.prefix_sum(w)
+        torch.cuda.synchronize()
+        assert torch.equal(got, full)
+    del w, got, full, first, state
+    n = (1 << 26) + 4097
+    announce("scan int64 n=%d (three launches)" % n)
+    v = torch.randint(-5, 6, (n,), device="cuda", generator=g, dtype=torch.int64)
+    v[4095::4096] -= v.view(-1)[: (n // 4096) * 4096].view(-1, 4096).sum(1) + 1   # every range sums to -1
+    assert torch.equal(ops.prefix_sum_i64(v), torch.cumsum(v, 0))
+
+
+def test_chained_scan_ignores_what_the_workspace_held():
+    """A workspace need not be initialised, and what memory holds is rarely random: words left by
+    index arrays, counts and their sums are small integers, as are the tags 1, 2, 3 ... that a
+    launch counter would hand out.  The chained kernel must not take any of it for a range sum
+    published in its own launch."""
+    import ctypes
     from gear_amd import _cabi
     lib = _cabi.load()
-    x = torch.zeros(16, dtype=torch.int64, device="cuda")
-    n = (1 << 26) + 1
-    ws = torch.zeros(lib.gear_hip_scan_workspace_bytes(n), dtype=torch.uint8, device="cuda")
-    import ctypes
-    rc = lib.gear_hip_scan_i64(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(x.data_ptr()), n,
-                               ctypes.c_void_p(ws.data_ptr()), ws.numel(), None)
-    assert rc == -3
+    g = torch.Generator(device="cuda").manual_seed(5)
+    n = 5_852_911
+    w = torch.rand(n, device="cuda", generator=g)
+    nbytes = int(lib.gear_hip_scan_workspace_bytes(n))
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    out = torch.empty(n, dtype=torch.float64, device="cuda")
+
+    def scan():
+        rc = lib.gear_hip_scan_f32_f64(ctypes.c_void_p(w.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+                                       n, ctypes.c_void_p(ws.data_ptr()), ws.numel(),
+                                       ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0
+        torch.cuda.synchronize()
+        return out.clone()
+
+    expect = scan()                                     # zeroed workspace
+    words = ws.view(torch.int64)
+    sums = torch.cumsum(torch.randint(0, 1 << 20, (words.numel(),), device="cuda", generator=g,
+                                      dtype=torch.int64), 0)
+    patterns = {
+        "running sums of small integers": sums,
+        "0, 1, 2, ...": torch.arange(words.numel(), device="cuda", dtype=torch.int64),
+        "tags 1, 2, 3 ... of an earlier process": (torch.arange(words.numel(), device="cuda",
+                                                                dtype=torch.int64) // 3 % 64 + 1) << 22,
+        "all ones": torch.full((words.numel(),), -1, device="cuda", dtype=torch.int64),
+    }
+    for what, fill in patterns.items():
+        for rep in range(8):                            # several launches: several tags
+            words.copy_(fill)
+            announce("chained scan, workspace holds %s (%d)" % (what, rep))
+            assert torch.equal(scan(), expect), what
 
 
 @pytest.mark.parametrize("n", [4097, 1_000_000, 3_000_001])
