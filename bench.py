@@ -863,8 +863,11 @@ def run_scan(args):
             "torch_fill_f64_us": timed_us(lambda: ybuf.fill_(1.0)),
             "torch_cumsum_f64_us": timed_us(lambda: torch.cumsum(pri, 0, dtype=torch.float64, out=ybuf)),
             "what": "HIP events around 50 back-to-back launches each, same n"}
-    variant = {"": "chained single pass (default)", "1": "chained single pass", "0": "two launches",
-               "2": "ticketed look-back"}.get(os.environ.get("GEAR_HIP_SCAN_SINGLE_PASS", ""), "?")
+    forced = os.environ.get("GEAR_HIP_SCAN_SINGLE_PASS", "")
+    ranges = -(-n // 8192)     # what the library does at this size: see gear_amd/csrc/scan.hip
+    by_size = ("three launches (range sums, their prefix, scan)" if ranges > 16384 else
+               "two launches" if ranges > 4096 or forced == "0" else "chained single pass")
+    variant = "ticketed look-back" if forced == "2" else by_size + (" (default)" if forced == "" else "")
     return _line(n / (ms * 1e-3), "priorities/s", args, ms,
                  "scan: fp64 prefix sum of %d fp32 priorities, %s" % (n, variant),
                  {"bound": "hbm", "kernel": "prefix sum chain (" + variant + ")",
