@@ -109,3 +109,35 @@ def test_random_topk_sort_scatter(oracle, seed):
     ops.scatter(dw, _dev(uidx_np), _dev(uval), unique_indices=False)
     torch.cuda.synchronize()
     assert np.array_equal(dw.cpu().numpy(), oracle.scatter_f32(w.copy(), uidx_np, uval))
+
+
+@pytest.mark.parametrize("seed", [3, 8, 13])
+def test_random_entry_points_with_workspaces_full_of_leftovers(oracle, seed, monkeypatch):
+    """No entry point may depend on what its workspace held: every shared workspace is refilled
+    before each use with what recycled memory typically holds (running sums of small integers,
+    all ones, 0 1 2 ..., random words)."""
+    from gear_amd import ops
+    plain_get = ops._ws.get
+    uses = [0]
+
+    def leftover_get(tag, nbytes, device):
+        buf = plain_get(tag, nbytes, device)
+        words = buf[: buf.numel() // 8 * 8].view(torch.int64)
+        kind = uses[0] % 4
+        uses[0] += 1
+        if kind == 0:
+            words.copy_(torch.cumsum(torch.randint(0, 1 << 20, (words.numel(),), device=buf.device,
+                                                   dtype=torch.int64), 0))
+        elif kind == 1:
+            words.fill_(-1)
+        elif kind == 2:
+            words.copy_(torch.arange(words.numel(), device=buf.device, dtype=torch.int64))
+        else:
+            words.copy_(torch.randint(-2**62, 2**62, (words.numel(),), device=buf.device,
+                                      dtype=torch.int64))
+        return buf
+
+    monkeypatch.setattr(ops._ws, "get", leftover_get)
+    test_random_scan_search_sample(oracle, seed)
+    test_random_topk_sort_scatter(oracle, seed)
+    assert uses[0] > 0
