@@ -1,6 +1,6 @@
-"""GPU parity of the weighted sampler: fp64 prefix sum (both variants of the range scan and the
-tiled look-back scan for very long inputs), batched upper_bound search, importance weights, through
-the C ABI against the CPU oracle."""
+"""GPU parity of the weighted sampler: fp64 prefix sum (the chained, two-launch and three-launch
+forms of the range scan and the tiled look-back scan kept for comparisons), batched upper_bound
+search, importance weights, through the C ABI against the CPU oracle."""
 import os
 
 import numpy as np
