@@ -15,9 +15,11 @@
 //             order: every entry above T and the first `need` entries equal to T (ties go to the
 //             smaller index).
 // Levels 1, 2, count and write walk the candidate lists (about 2 % of the input) when the hint
-// held and no list overflowed; otherwise each of them streams the priorities again (count then
-// rebuilds the lists with the exact threshold, write re-reads if those overflow too).  The hint
-// only decides which of the two it is, never the result.
+// held; a wave whose list overflowed (clustered maxima, masses of equal priorities) reads its own
+// range of the priorities again instead, in each of them (count then rebuilds its list with the
+// exact threshold, write re-reads if that overflows too).  When the hint did not hold (fewer
+// than k candidates: the picked bin lies below it) every wave does.  The hint only decides
+// which of the two it is, never the result.
 // Value order (k <= 131072): write leaves the selection as (key, index, segment) in index order
 // and puts the entries equal to T straight at the tail of the output; the level-0 histogram says
 // where every bin starts in value order, bins that start in the same stretch of output places
@@ -57,6 +59,7 @@ static_assert((1ll << 32 >> kLowShift) + kMidBins + (1ll << (32 - kMaxBinBits)) 
 // reads the whole input again.
 constexpr int kMaxSamplesPerThread = 32;
 constexpr uint32_t kNoLists = 0xffffffffu;   // hint_bin: level 0 writes no candidate lists
+constexpr uint32_t kListFull = 0xffffffffu;  // wave_listed: the wave's list overflowed, the wave reads its range instead
 constexpr int64_t kBucketMaxK = 131072;      // value order by buckets up to this k
 constexpr int kSortThreads = 1024;           // segment sort workgroup
 constexpr int kSmallGroup = 256;             // groups up to this size are ranked directly
@@ -97,8 +100,8 @@ __device__ __forceinline__ uint32_t bin_hi_key(const BinMap &m, uint32_t bin) {
 struct State {
   uint32_t prefix[3];  // level-0 bin, level-1 digit, threshold key
   uint32_t k_rem[3];   // entries still to take from the bin picked at that level
-  uint32_t overflow;   // a level-0 list overflowed (or no lists were asked for)
-  uint32_t overflow2;  // a list rebuilt by count overflowed: write re-reads the priorities
+  uint32_t overflow;   // no lists were asked for: every level reads the priorities
+  uint32_t overflow2;  // (unused)
   uint32_t hint_bin;   // candidates are the entries whose level-0 bin is >= this
   uint32_t full;       // levels 1, 2, count stream the priorities instead of the lists
   uint32_t lo0, hi0;   // smallest and largest key of the picked level-0 bin
@@ -411,6 +414,45 @@ __device__ __forceinline__ void stream_range_tagged(const float *__restrict__ p,
   }
 }
 
+// The same range as rows of 64 consecutive elements, one per lane: f(i, v, valid) for the lane's
+// element i of every row (all lanes call), rows in index order.  For a wave that stores something
+// per element: the lanes' stores then fall side by side.
+template <typename F>
+__device__ __forceinline__ void stream_rows(const float *__restrict__ p, int64_t begin, int64_t end,
+                                            int lane, F f) {
+  if (begin >= end) return;
+  auto load_step = [&](int64_t s0, float (&q)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t i = s0 + j * kWave + lane;
+      q[j] = i < end ? p[i] : 0.0f;
+    }
+  };
+  float q[kAhead][4];
+#pragma unroll
+  for (int a = 0; a < kAhead; ++a) load_step(begin + (int64_t)a * kStep, q[a]);
+  for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
+    float qn[kAhead][4];
+    const int64_t s1 = s0 + kAhead * kStep;
+    if (s1 < end) {
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) load_step(s1 + (int64_t)a * kStep, qn[a]);
+    }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t r0 = s0 + (int64_t)a * kStep + j * kWave;
+        if (r0 < end) f(r0 + lane, q[a][j], r0 + lane < end);
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q[a][j] = qn[a][j];
+  }
+}
+
 // Appends the lane's selected entries (sel[j], in element order) to the wave's list in index
 // order.  `listed` counts every candidate seen, also the ones that no longer fit (wave-uniform).
 __device__ __forceinline__ void list_append(uint64_t *list, int list_cap, int &listed,
@@ -615,10 +657,15 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
     // the wave's queue: ordered by index (every entry counts the smaller ones), binned, listed
     const uint32_t m_all = nq;
     const uint32_t m = m_all < (uint32_t)cap ? m_all : (uint32_t)cap;
+    const bool given_up = m_all > (uint32_t)cap;  // the list is not used: its entries are only binned
     for (uint32_t i = lane; i < m; i += kWave) {
       const uint64_t mine = wq[i];
       const uint32_t index = (uint32_t)mine;
       uint32_t r = 0;
+      if (given_up) {
+        count_add(h, bin_of(map, order_key(__uint_as_float((uint32_t)(mine >> 32)))), true);
+        continue;
+      }
       if (m <= kRankAll) {
         const uint32_t m8 = m & ~7u;
         for (uint32_t j = 0; j < m8; j += 8) {  // eight LDS reads in flight
@@ -652,8 +699,9 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
       list[r] = ((uint64_t)key << 32) | index;
     }
     if (lane == 0) {
-      wave_listed[gw] = m;
-      if (m_all > (uint32_t)cap) state->overflow = 1u;  // same value from every overflowing wave
+      // a wave whose list overflowed (clustered maxima, masses of equal priorities) says so:
+      // the later launches read its range of the priorities again, its range only
+      wave_listed[gw] = m_all > (uint32_t)cap ? kListFull : m;
     }
   }
   __syncthreads();
@@ -683,7 +731,9 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
   // before the histogram is walked (used only when the lists are in use)
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   const uint64_t *list = lists + gw * list_cap;
-  const int m_pre = (int)wave_listed[gw];
+  // (the same word in every lane: said so, the branches on it are taken by whole waves)
+  const uint32_t m_raw = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave_listed[gw]);
+  const int m_pre = (int)m_raw;
   const uint64_t ent_pre = list[lane];
   uint32_t lo, hi;  // the keys that are counted
   int shift;        // digit = (key - lo) >> shift
@@ -720,7 +770,8 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
     }
   }
   __syncthreads();
-  if (!full) {
+  // a wave whose list overflowed reads its own range again, the others walk their lists
+  if (!full && m_raw != kListFull) {
     const int m = m_pre;
     for (int c0 = 0; c0 < m; c0 += kWave) {
       if (c0 + lane < m) {
@@ -762,10 +813,12 @@ __global__ __launch_bounds__(kThreads) void count_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   uint64_t *list = lists + gw * list_cap;
-  const int m_pre = (int)wave_listed[gw];  // asked for before the pick; used with the lists only
+  // (the same word in every lane: said so, the branches on it are taken by whole waves)
+  const uint32_t m_raw = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave_listed[gw]);
+  const int m_pre = (int)m_raw;
   const uint64_t ent_pre = list[lane];
   const uint32_t lo0 = state->lo0, hi0 = state->hi0, digit1 = state->prefix[1];
-  const bool full = state->full != 0u;
+  const bool full = state->full != 0u || m_raw == kListFull;  // this wave reads its range
   const Pick r = pick_bin<kBinsR>(state->k_rem[1], hist2, nullptr);
   const uint32_t thr = lo0 + (digit1 << level1_shift(bits_of(hi0 - lo0))) + r.bin;
   if (blockIdx.x == 0 && tid == 0) {
@@ -803,8 +856,7 @@ __global__ __launch_bounds__(kThreads) void count_kernel(
       }
       list_append(list, list_cap, listed, overflow, sel, key, e0, lt_mask);
     });
-    if (lane == 0) wave_listed[gw] = (uint32_t)listed;
-    if (overflow && lane == 0) state->overflow2 = 1u;
+    if (lane == 0) wave_listed[gw] = overflow ? kListFull : (uint32_t)listed;
   }
   const int64_t w = wave_sum((int64_t)(((uint64_t)gt << 32) | (uint64_t)eq));
   if (lane == 0) {
@@ -839,11 +891,13 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   const uint64_t *list = lists + gw * list_cap;
-  const int m_pre = (int)wave_listed[gw];
+  // (the same word in every lane: said so, the branch on it is taken by whole waves)
+  const uint32_t m_raw = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave_listed[gw]);
+  const int m_pre = (int)m_raw;
   const uint64_t ent_pre = list[lane];
   const uint32_t thr = state->prefix[2];
   const uint32_t need_eq = state->k_rem[2];
-  const bool reread = state->full != 0u && state->overflow2 != 0u;
+  const bool reread = m_raw == kListFull;
   const BinMap map = state->map;
 
   // counts of the workgroups before this one (at most kMaxBlocks), then of the waves before
@@ -919,31 +973,20 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
   const float thr_f = key_to_float(thr);
   const int64_t begin = gw * wave_len;
   const int64_t end = begin + wave_len < n ? begin + wave_len : n;
-  stream_range(p, begin, end, lane, [&](int64_t e0, const float q[4]) {
-    int s = 0;  // packed counts of the lane's four entries: greater << 16 | equal
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (e0 + j < end) s += q[j] > thr_f ? (1 << 16) : (q[j] == thr_f ? 1 : 0);
-    if (wave_ballot(s != 0) == 0ull) return;
-    // nothing of the step is selected once the ties needed are placed and no entry is above T
-    if (eq_run >= need_eq && wave_ballot((s >> 16) != 0) == 0ull) return;
-    const int inc = wave_inclusive_sum(s);
-    const int total = wave_read_lane(inc, kWave - 1);
-    const int before = inc - s;
-    uint32_t g = gt_run + ((uint32_t)before >> 16);
-    uint32_t e = eq_run + ((uint32_t)before & 0xffffu);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bool valid = e0 + j < end;
-      const bool is_gt = valid && q[j] > thr_f, is_eq = valid && q[j] == thr_f;
-      const bool selected = is_gt || (is_eq && e < need_eq);
-      emit(selected, is_eq, g + (e < need_eq ? e : need_eq), e, (uint32_t)(e0 + j),
-           is_gt ? order_key(q[j]) : thr, std::true_type{}, q[j]);
-      g += is_gt;
-      e += is_eq;
-    }
-    gt_run += (uint32_t)total >> 16;
-    eq_run += (uint32_t)total & 0xffffu;
+  // (rows of 64: the stores of a row's selected entries fall side by side -- a wave that comes
+  // here is one whose list overflowed, and such a wave often selects most of its range)
+  stream_rows(p, begin, end, lane, [&](int64_t i, float v, bool valid) {
+    const bool is_gt = valid && v > thr_f, is_eq = valid && v == thr_f;
+    const uint64_t bg = wave_ballot(is_gt), be = wave_ballot(is_eq);
+    // nothing of the row is selected once the ties needed are placed and no entry is above T
+    if (bg == 0ull && (be == 0ull || eq_run >= need_eq)) return;
+    const uint32_t g = gt_run + (uint32_t)__popcll(bg & lt_mask);
+    const uint32_t e = eq_run + (uint32_t)__popcll(be & lt_mask);
+    const bool selected = is_gt || (is_eq && e < need_eq);
+    emit(selected, is_eq, g + (e < need_eq ? e : need_eq), e, (uint32_t)i,
+         is_gt ? order_key(v) : thr, std::true_type{}, v);
+    gt_run += (uint32_t)__popcll(bg);
+    eq_run += (uint32_t)__popcll(be);
   });
 }
 
