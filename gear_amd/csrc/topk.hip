@@ -565,11 +565,10 @@ __device__ __forceinline__ void count_add(uint32_t *cnt, uint32_t d, bool valid)
 // Every entry is counted in its level-0 bin (LDS histogram, flushed with atomics); the
 // candidates -- entries at or above the hint, about one in fifty -- are also listed per wave, in
 // index order, as key << 32 | index.  While streaming, a candidate is only dropped into the
-// wave's queue in LDS (value | index, in the order of arrival: nearly every wave step holds one
-// or two candidates, so whatever is done per candidate there is paid per step); after the
-// stream the wave orders its queue by index, bins the candidates and writes the list, all lanes
-// busy.  A candidate that finds the queue full is binned at once and the lists are given up.
-constexpr uint32_t kRankAll = 160;  // queues up to this length are ordered by comparing every pair
+// wave's queue in LDS (value | index, at its place in index order: nearly every wave step holds
+// one or two candidates, so whatever is done per candidate there is paid per step); after the
+// stream the wave bins the candidates of its queue and writes the list, all lanes busy.  A
+// candidate that finds the queue full is binned at once and the wave's list is given up.
 constexpr int kQueueCap = 512;  // candidates per wave held in LDS; longer lists overflow
 
 __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restrict__ p, int64_t n,
@@ -632,13 +631,17 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
       // everything else goes to its coarse bin right away
       if (valid && !cand) atomicAdd(&h[order_key(q[j]) >> low_shift], 1u);
     }
-    uint64_t with;  // lanes that still hold a candidate; a lane rarely has two: one round
-    while ((with = wave_ballot(rem != 0u)) != 0ull) {
+    // The candidates of the step enter the queue in index order.  Mostly no lane holds more
+    // than one: the lanes' candidates, lanes in order, are in index order as they are.  Else a
+    // lane's place follows from the candidates of the lanes before it (up to four each: a
+    // ballot per bit of the count).  A candidate that finds the queue full is binned at once.
+    const uint64_t with = wave_ballot(rem != 0u);
+    if (with == 0ull) return;
+    if (wave_ballot((rem & (rem - 1u)) != 0u) == 0ull) {
       bool over = false;
       uint32_t over_bin = 0u;
       if (rem != 0u) {
         const int j = __ffs((int)rem) - 1;
-        rem &= rem - 1u;
         const float x = j == 0 ? q[0] : (j == 1 ? q[1] : (j == 2 ? q[2] : q[3]));
         const uint32_t at = nq + (uint32_t)__popcll(with & lt_mask);
         if (at < (uint32_t)cap) {
@@ -649,54 +652,40 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
         }
       }
       nq += (uint32_t)__popcll(with);
-      // the queue is full (the lists are given up): masses of equal priorities share a bin
       if (nq > (uint32_t)cap) count_add(h, over_bin, over);
+    } else {
+      const int nc = __popc(rem);
+      const uint64_t b0 = wave_ballot((nc & 1) != 0), b1 = wave_ballot((nc & 2) != 0),
+                     b2 = wave_ballot((nc & 4) != 0);
+      uint32_t at = nq + (uint32_t)(__popcll(b0 & lt_mask) + 2 * __popcll(b1 & lt_mask) +
+                                    4 * __popcll(b2 & lt_mask));
+      nq += (uint32_t)(__popcll(b0) + 2 * __popcll(b1) + 4 * __popcll(b2));
+      const bool spills = nq > (uint32_t)cap;  // masses of equal priorities share a bin
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool c = ((rem >> j) & 1u) != 0u;
+        const bool over = c && at >= (uint32_t)cap;
+        if (c && !over) wq[at] = ((uint64_t)__float_as_uint(q[j]) << 32) | (uint32_t)(e0 + j);
+        if (spills) count_add(h, over ? bin_of(map, order_key(q[j])) : 0u, over);
+        at += c ? 1u : 0u;
+      }
     }
   });
   if (want_lists) {
-    // the wave's queue: ordered by index (every entry counts the smaller ones), binned, listed
+    // the wave's queue, in index order, is binned and becomes the wave's list, all lanes busy (an
+    // overflowed one is only binned: the later launches read the wave's range instead)
     const uint32_t m_all = nq;
     const uint32_t m = m_all < (uint32_t)cap ? m_all : (uint32_t)cap;
-    const bool given_up = m_all > (uint32_t)cap;  // the list is not used: its entries are only binned
+    const bool given_up = m_all > (uint32_t)cap;
     for (uint32_t i = lane; i < m; i += kWave) {
       const uint64_t mine = wq[i];
-      const uint32_t index = (uint32_t)mine;
-      uint32_t r = 0;
-      if (given_up) {
-        count_add(h, bin_of(map, order_key(__uint_as_float((uint32_t)(mine >> 32)))), true);
-        continue;
-      }
-      if (m <= kRankAll) {
-        const uint32_t m8 = m & ~7u;
-        for (uint32_t j = 0; j < m8; j += 8) {  // eight LDS reads in flight
-          uint32_t x[8];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) x[u] = (uint32_t)wq[j + u];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) r += x[u] < index;
-        }
-        for (uint32_t j = m8; j < m; ++j) r += (uint32_t)wq[j] < index;
-      } else {
-        // A long queue: it holds the steps of the stream one after the other, and only inside
-        // a step the order of arrival (every lane's first candidate, then the second ones) is
-        // not the order of the indices: the entry looks at its neighbours of the same step.
-        const uint32_t first = (uint32_t)begin;  // a multiple of kStep
-        const uint32_t step = (index - first) / (uint32_t)kStep;
-        r = i;
-        for (uint32_t j = i; j-- > 0u;) {
-          const uint32_t other = (uint32_t)wq[j];
-          if ((other - first) / (uint32_t)kStep != step) break;
-          r -= other > index;
-        }
-        for (uint32_t j = i + 1; j < m; ++j) {
-          const uint32_t other = (uint32_t)wq[j];
-          if ((other - first) / (uint32_t)kStep != step) break;
-          r += other < index;
-        }
-      }
       const uint32_t key = order_key(__uint_as_float((uint32_t)(mine >> 32)));
-      atomicAdd(&h[bin_of(map, key)], 1u);
-      list[r] = ((uint64_t)key << 32) | index;
+      if (given_up) {
+        count_add(h, bin_of(map, key), true);
+      } else {
+        atomicAdd(&h[bin_of(map, key)], 1u);
+        list[i] = ((uint64_t)key << 32) | (uint32_t)mine;
+      }
     }
     if (lane == 0) {
       // a wave whose list overflowed (clustered maxima, masses of equal priorities) says so:
