@@ -305,8 +305,9 @@ int gear_hip_sort_i64(const int64_t *keys_in, int64_t *keys_out, const int64_t *
  * values_out may be NULL.  1 <= k <= n < 2^31.
  * The priorities are normally read once: a sample of 2048 of them places a bound safely below
  * the k-th largest, the one pass over the array lists everything above the bound, and the exact
- * selection runs on those lists.  Where the bound fails or a list overflows (clustered maxima,
- * masses of ties) the later steps read the array again; the result is the same either way.
+ * selection runs on those lists.  Where a list overflows (clustered maxima, masses of ties) the
+ * later steps read that part of the array again, where the bound fails all of it; the result is
+ * the same either way.
  * workspace: gear_hip_topk_workspace_bytes(n, k) bytes on the device, 256-byte aligned; its
  * contents need not be initialised (the call clears what it needs on `stream`). */
 size_t gear_hip_topk_workspace_bytes(int64_t n, int64_t k);
