@@ -501,9 +501,9 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
     // memory delivers ranges anyway) makes the ranges arrive in order: early ranges are being
     // written while late ones are still being read.  The wait is bounded by first_wave * stagger.
     if (stagger > 0 && blockIdx.x < (unsigned)first_wave) {
-      const unsigned long long until =
-          wall_clock64() + (((unsigned long long)blockIdx.x * (unsigned)stagger) >> 10);
-      while (wall_clock64() < until) __builtin_amdgcn_s_sleep(1);
+      const unsigned long long until = (unsigned long long)wall_clock64() +
+                                       (((unsigned long long)blockIdx.x * (unsigned)stagger) >> 10);
+      while ((unsigned long long)wall_clock64() < until) __builtin_amdgcn_s_sleep(1);
     }
   }
   In f[geo::kEPT];
