@@ -512,7 +512,7 @@ def run_config2(args):
     return _line(B / (ms * 1e-3), "draws/s", args, ms,
                  "config2: 1e6 fp32 priorities -> fp64 prefix (one chained single-pass launch), 4096 "
                  "draws, importance weights",
-                 {"bound": "hbm", "kernel": "scan_ranges_kernel<float, double, 4, NR, true>", "achieved": alg / (sms * 1e-3) / 1e9,
+                 {"bound": "hbm", "kernel": "scan_ranges_kernel<float, double, double, G, kChained> (one launch: the chained prefix sum)", "achieved": alg / (sms * 1e-3) / 1e9,
                   "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / (sms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                   "avg_launch_ms": sms, "algorithmic_bytes": alg, "traffic": None},
                  dict(_graph_extra(B, "draws/s", ms_graph),
@@ -818,7 +818,7 @@ def _calibrate_copy(torch, ops):
 def run_scan(args):
     """One kernel chain on its own: fp64 prefix sum of --n fp32 priorities.  The variant follows
     GEAR_HIP_SCAN_SINGLE_PASS (unset or 1: chained single pass, 0: range sums + scan in two
-    launches, 2: ticketed look-back)."""
+    launches)."""
     import numpy as np
     import torch
     from gear_amd import ops
@@ -867,7 +867,7 @@ def run_scan(args):
     ranges = -(-n // 8192)     # what the library does at this size: see gear_amd/csrc/scan.hip
     by_size = ("three launches (range sums, their prefix, scan)" if ranges > 16384 else
                "two launches" if ranges > 4096 or forced == "0" else "chained single pass")
-    variant = "ticketed look-back" if forced == "2" else by_size + (" (default)" if forced == "" else "")
+    variant = by_size + (" (default)" if forced == "" else "")
     return _line(n / (ms * 1e-3), "priorities/s", args, ms,
                  "scan: fp64 prefix sum of %d fp32 priorities, %s" % (n, variant),
                  {"bound": "hbm", "kernel": "prefix sum chain (" + variant + ")",

@@ -311,17 +311,12 @@ Shape plan(int64_t num, int64_t max_region, int U) {
   return s;
 }
 
-// Measured on MI355X at the 2048 x 847 KB window shape: two vectors per thread (8 KiB per
-// workgroup, many small workgroups) with non-temporal stores moves 6.1 TB/s; four or eight
-// vectors per thread, or plain stores, stay between 5.1 and 5.7 TB/s.
-int pick_unroll() {
-  static int u = env_int("GEAR_HIP_GATHER_UNROLL", 2);
-  return (u == 2 || u == 4 || u == 8) ? u : 2;
-}
-int pick_nt() {
-  static int nt = env_int("GEAR_HIP_GATHER_NT", 2);
-  return nt == 0 ? 0 : 2;
-}
+// The one instantiation that is built: two vectors per thread (8 KiB per workgroup, many small
+// workgroups) with non-temporal stores.  Measured on MI355X at the 2048 x 847 KB window shape
+// that moves 6.1-6.3 TB/s; four or eight vectors per thread, or plain stores, stay between 5.1
+// and 5.7 TB/s, non-temporal loads change nothing.
+constexpr int kUnroll = 2;
+constexpr int kNt = 2;  // bit mask: 1 = non-temporal loads, 2 = non-temporal stores
 
 int fill_column(const gear_hip_column_desc &d, int64_t num, int U, ColumnArgs *out,
                 int64_t *blocks) {
@@ -348,63 +343,26 @@ int fill_column(const gear_hip_column_desc &d, int64_t num, int U, ColumnArgs *o
   return 0;
 }
 
-template <int U, int NT>
-int launch_subcopy_un(const GatherArgs &p, const ColumnArgs &col, int64_t blocks, hipStream_t st) {
-  subcopy_kernel<U, NT><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, col);
+int launch_subcopy(const GatherArgs &p, const ColumnArgs &col, int64_t blocks, hipStream_t st) {
+  subcopy_kernel<kUnroll, kNt><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, col);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
 
-template <int U, int NT>
-int launch_multi_un(const GatherArgs &p, const MultiArgs &m, int64_t blocks, hipStream_t st) {
-  subcopy_multi_kernel<U, NT><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, m);
+int launch_multi(const GatherArgs &p, const MultiArgs &m, int64_t blocks, hipStream_t st) {
+  subcopy_multi_kernel<kUnroll, kNt><<<dim3((unsigned)blocks), dim3(kBlock), 0, st>>>(p, m);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
-}
-
-template <int MODE, int U, int NT>
-int launch_slices_un(const GatherArgs &p, uint8_t *dst, const Shape &s, hipStream_t st) {
-  slices_kernel<MODE, U, NT><<<dim3((unsigned)s.blocks), dim3(kBlock), 0, st>>>(p, dst, s.cps,
-                                                                              s.tg_shift);
-  GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  return 0;
-}
-
-// picks the instantiation for the (unroll, non-temporal) pair chosen at run time
-#define GEARHIP_DISPATCH_U_NT(U, NT, CALL)                          \
-  do {                                                              \
-    if ((NT) == 0) {                                                \
-      if ((U) == 8) return CALL(8, 0);                              \
-      if ((U) == 4) return CALL(4, 0);                              \
-      return CALL(2, 0);                                            \
-    }                                                               \
-    if ((U) == 8) return CALL(8, 2);                                \
-    if ((U) == 4) return CALL(4, 2);                                \
-    return CALL(2, 2);                                              \
-  } while (0)
-
-int launch_subcopy(const GatherArgs &p, const ColumnArgs &col, int64_t blocks, int U, int nt,
-                   hipStream_t st) {
-#define CALL_(UU, NN) launch_subcopy_un<UU, NN>(p, col, blocks, st)
-  GEARHIP_DISPATCH_U_NT(U, nt, CALL_);
-#undef CALL_
-}
-
-int launch_multi(const GatherArgs &p, const MultiArgs &m, int64_t blocks, int U, int nt,
-                 hipStream_t st) {
-#define CALL_(UU, NN) launch_multi_un<UU, NN>(p, m, blocks, st)
-  GEARHIP_DISPATCH_U_NT(U, nt, CALL_);
-#undef CALL_
 }
 
 template <int MODE>
 int launch_slices(const GatherArgs &p, uint8_t *dst, int64_t max_len, hipStream_t st) {
-  const int U = pick_unroll(), nt = pick_nt();
-  const Shape s = plan(p.num, max_len, U);
+  const Shape s = plan(p.num, max_len, kUnroll);
   if (s.blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
-#define CALL_(UU, NN) launch_slices_un<MODE, UU, NN>(p, dst, s, st)
-  GEARHIP_DISPATCH_U_NT(U, nt, CALL_);
-#undef CALL_
+  slices_kernel<MODE, kUnroll, kNt><<<dim3((unsigned)s.blocks), dim3(kBlock), 0, st>>>(
+      p, dst, s.cps, s.tg_shift);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
 }
 
 }  // namespace
@@ -430,14 +388,14 @@ extern "C" int gear_hip_subcopy(const void *src, void *dst, int64_t num, const i
   d.dst_stride = dst_stride;
   d.pad_head = pad_head;
   d.zero_fill = zero_fill;
-  const int U = pick_unroll();
+  const int U = kUnroll;
   ColumnArgs col;
   int64_t blocks = 0;
   int rc = fill_column(d, num, U, &col, &blocks);
   if (rc) return rc;
   if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
   GatherArgs p{static_cast<const uint8_t *>(src), num, idxs, tss, lens, traj_stride, 0, 0, 0};
-  return launch_subcopy(p, col, blocks, U, pick_nt(), as_stream(stream));
+  return launch_subcopy(p, col, blocks, as_stream(stream));
 }
 
 extern "C" int gear_hip_subcopy_multi(const void *src, int64_t num, const int64_t *idxs,
@@ -458,7 +416,7 @@ extern "C" int gear_hip_subcopy_multi_checked(const void *src, int64_t num, cons
     return GEAR_HIP_EINVAL;
   if (num == 0 || ncols == 0) return 0;
   if (!src || !idxs || !tss || !lens || !cols || traj_stride < 0) return GEAR_HIP_EINVAL;
-  const int U = pick_unroll();
+  const int U = kUnroll;
   MultiArgs m;
   m.ncols = ncols;
   int64_t total = 0;
@@ -473,7 +431,7 @@ extern "C" int gear_hip_subcopy_multi_checked(const void *src, int64_t num, cons
   if (total >= 0x7fffffffll) return GEAR_HIP_ERANGE;
   GatherArgs p{static_cast<const uint8_t *>(src), num,        idxs, tss, lens, traj_stride, 0,
                capacity,                          trajectory_length};
-  return launch_multi(p, m, total, U, pick_nt(), as_stream(stream));
+  return launch_multi(p, m, total, as_stream(stream));
 }
 
 extern "C" int gear_hip_vcopy(const void *src, void *dst, int64_t num,

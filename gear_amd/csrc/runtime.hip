@@ -25,7 +25,11 @@ extern "C" int gear_hip_set_device(int device_id) {
   int current = -1;
   GEARHIP_CHECK(hipGetDevice(&current));
   if (current != device_id) GEARHIP_CHECK(hipSetDevice(device_id));
-  return scan_static_init();
+  // Warm-up of the allocation-free prefix sum (address of its static array, its ordering event):
+  // best effort -- a failure here must not fail device selection for callers that never use
+  // that entry point, which reports the error itself when it is called.
+  if (scan_static_init() != 0) (void)hipGetLastError();
+  return 0;
 }
 
 extern "C" int gear_hip_device_count(int *count) {
@@ -46,6 +50,7 @@ extern "C" const char *gear_hip_error_string(int code) {
     case GEAR_HIP_EWORKSPACE: return "gear_hip: workspace missing or too small";
     case GEAR_HIP_ERANGE: return "gear_hip: size out of the supported range";
     case GEAR_HIP_EALIGN: return "gear_hip: pointer is not sufficiently aligned";
+    case GEAR_HIP_ENOTREADY: return "gear_hip: set-up for this call has not run and cannot run now";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);

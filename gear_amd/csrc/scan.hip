@@ -22,13 +22,9 @@
 //  * beyond that: three launches -- range_sum_kernel, range_prefix_kernel (ONE workgroup scans the
 //    range sums in a fixed order) and scan_ranges_kernel<kPrefixed>, which finds the sum of all
 //    earlier ranges in one word.  Same bits on every run, and for the rescan of a suffix.
-//  * scan_kernel, the tiled decoupled look-back (aggr[t] = sum of tile t alone, incl[t] = sum of
-//    tiles 0..t; wave 0 looks back 64 predecessors at a time, ballots pick the nearest published
-//    inclusive value; tile numbers come from an atomic ticket), runs only when asked for
-//    (GEAR_HIP_SCAN_SINGLE_PASS=2, for comparisons): what it adds up depends on which
-//    predecessors had published what, so two runs can differ in the last bit.
 #include <atomic>
 #include <chrono>
+#include <mutex>
 #include <random>
 #include <type_traits>
 
@@ -38,8 +34,7 @@ namespace gearhip {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kRows = 4;
-constexpr uint64_t kEmpty = ~0ull;  // no fp64 sum of fp32 values has this bit pattern (fp64 scans only)
+constexpr int kMinRange = 2048;  // elements of the smallest range (fp32, 2 granules per thread)
 constexpr size_t kHeaderBytes = 256;
 
 template <typename Acc> struct Bits;
@@ -52,30 +47,6 @@ template <> struct Bits<int64_t> {
   static __device__ __forceinline__ int64_t from(uint64_t b) { return (int64_t)b; }
 };
 
-template <typename In, int VE> struct InVec;
-template <> struct InVec<float, 4> {
-  typedef float type __attribute__((ext_vector_type(4), aligned(4)));
-};
-template <> struct InVec<int64_t, 2> {
-  typedef int64_t type __attribute__((ext_vector_type(2), aligned(8)));
-};
-template <typename Acc> struct OutVec2;
-// result vectors are stored with their natural alignment (the launcher checks the pointer)
-template <> struct OutVec2<double> {
-  typedef double type __attribute__((ext_vector_type(2)));
-};
-template <> struct OutVec2<int64_t> {
-  typedef int64_t type __attribute__((ext_vector_type(2)));
-};
-template <> struct OutVec2<float> {
-  typedef float type __attribute__((ext_vector_type(2)));
-};
-
-// Writes the VE consecutive results of every lane of a wave (a contiguous slice of 64*VE
-// elements starting at e_wave) so that each store instruction covers one contiguous run:
-// non-temporal stores only reach full bandwidth when a wave writes whole cache lines.  With
-// 16 bytes per lane the lanes already do; with 32 bytes per lane (fp64 results of a float4) the
-// slice takes a detour through a wave-private LDS row.
 // Results that fit the caches are stored normally (the search that follows reads them back);
 // larger ones stream past the caches with non-temporal stores.
 template <typename V>
@@ -84,162 +55,6 @@ __device__ __forceinline__ void store_vec(V *p, V v, bool nt) {
     __builtin_nontemporal_store(v, p);
   else
     *p = v;
-}
-
-template <typename Out, int VE>
-__device__ __forceinline__ void store_slice(Out *__restrict__ out, int64_t e_wave, int64_t n,
-                                            const Out (&v)[VE], Out *stage_row, int lane) {
-  const bool nt = n * (int64_t)sizeof(Out) > (32ll << 20);
-  typedef typename OutVec2<Out>::type out_vec2;
-  constexpr int kLaneBytes = VE * (int)sizeof(Out);
-  const int64_t e0 = e_wave + (int64_t)lane * VE;
-  if (e_wave + (int64_t)kWave * VE > n) {  // ragged end of the input
-#pragma unroll
-    for (int j = 0; j < VE; ++j)
-      if (e0 + j < n) out[e0 + j] = v[j];
-    return;
-  }
-  if (kLaneBytes <= 16) {
-#pragma unroll
-    for (int j = 0; j < VE; j += 2) {
-      out_vec2 o;
-      o[0] = v[j];
-      o[1] = v[j + 1];
-      store_vec(reinterpret_cast<out_vec2 *>(out + e0 + j), o, nt);
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < VE; ++j) stage_row[lane * VE + j] = v[j];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int h = 0; h < VE / 2; ++h) {
-      out_vec2 o;
-      o[0] = stage_row[h * 2 * kWave + 2 * lane];
-      o[1] = stage_row[h * 2 * kWave + 2 * lane + 1];
-      store_vec(reinterpret_cast<out_vec2 *>(out + e_wave + (int64_t)h * 2 * kWave + 2 * lane), o,
-                nt);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  }
-}
-
-__global__ void scan_init_kernel(uint32_t *ticket, uint64_t *desc, int64_t words) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i == 0) *ticket = 0u;
-  if (i < words) desc[i] = kEmpty;
-}
-
-template <typename In, typename Acc, typename Out, int VE>
-__global__ __launch_bounds__(kBlock) void scan_kernel(const In *__restrict__ in,
-                                                      Out *__restrict__ out, int64_t n,
-                                                      uint32_t *ticket, uint64_t *aggr,
-                                                      uint64_t *incl) {
-  constexpr int kTileElems = kRows * kBlock * VE;
-  constexpr int kWaves = kBlock / kWave;
-  typedef typename InVec<In, VE>::type in_vec;
-  __shared__ Acc wtot[kRows][kWaves];
-  __shared__ Out stage[kWaves][kWave * VE];
-  __shared__ Acc s_excl;
-  __shared__ uint32_t s_tile;
-
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
-  if (tid == 0) s_tile = atomicAdd(ticket, 1u);
-  __syncthreads();
-  const int64_t tile = s_tile;
-  const int64_t base = tile * kTileElems;
-
-  Acc x[kRows][VE];
-  Acc s[kRows];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int64_t e0 = base + ((int64_t)r * kBlock + tid) * VE;
-    if (e0 + VE <= n) {
-      const in_vec v = *reinterpret_cast<const in_vec *>(in + e0);
-#pragma unroll
-      for (int j = 0; j < VE; ++j) x[r][j] = (Acc)v[j];
-    } else {
-#pragma unroll
-      for (int j = 0; j < VE; ++j) x[r][j] = (e0 + j < n) ? (Acc)in[e0 + j] : (Acc)0;
-    }
-#pragma unroll
-    for (int j = 1; j < VE; ++j) x[r][j] += x[r][j - 1];
-    s[r] = x[r][VE - 1];
-  }
-
-  Acc wexcl[kRows];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const Acc inc = wave_inclusive_sum(s[r]);
-    wexcl[r] = wave_shift_up1(inc);
-    if (lane == kWave - 1) wtot[r][wave] = inc;
-  }
-  __syncthreads();
-
-  Acc tile_total = (Acc)0;
-  Acc mybase[kRows];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    Acc acc = tile_total;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      if (w == wave) mybase[r] = acc + wexcl[r];
-      acc += wtot[r][w];
-    }
-    tile_total = acc;
-  }
-
-  if (wave == 0) {
-    Acc excl = (Acc)0;
-    if (tile == 0) {
-      if (lane == 0) store_agent(&incl[0], Bits<Acc>::to(tile_total));
-    } else {
-      if (lane == 0) store_agent(&aggr[tile], Bits<Acc>::to(tile_total));
-      int64_t look = tile - 1;
-      while (true) {
-        const int64_t idx = look - lane;
-        uint64_t vi = kEmpty, va = kEmpty;
-        if (idx >= 0) {
-          vi = load_agent(&incl[idx]);
-          if (vi == kEmpty) va = load_agent(&aggr[idx]);
-        }
-        const bool has_incl = (idx < 0) || (vi != kEmpty);
-        const bool ready = has_incl || (va != kEmpty);
-        const uint64_t bi = wave_ballot(has_incl), br = wave_ballot(ready);
-        const int first = bi ? (__ffsll((unsigned long long)bi) - 1) : kWave;
-        const uint64_t need = first >= 63 ? ~0ull : ((2ull << first) - 1ull);
-        if ((br & need) != need) {
-          __builtin_amdgcn_s_sleep(1);
-          continue;
-        }
-        Acc c = (Acc)0;
-        if (lane < first)
-          c = Bits<Acc>::from(va);
-        else if (lane == first && idx >= 0)
-          c = Bits<Acc>::from(vi);
-        excl += wave_sum(c);
-        if (first < kWave) break;
-        look -= kWave;
-      }
-      if (lane == 0) store_agent(&incl[tile], Bits<Acc>::to(excl + tile_total));
-    }
-    if (lane == 0) s_excl = excl;
-  }
-  __syncthreads();
-  const Acc excl = s_excl;
-
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const Acc b = excl + mybase[r];
-    Out o[VE];
-#pragma unroll
-    for (int j = 0; j < VE; ++j) o[j] = (Out)(b + x[r][j]);
-    store_slice<Out, VE>(out, base + ((int64_t)r * kBlock + wave * kWave) * VE, n, o, stage[wave],
-                         lane);
-  }
 }
 
 // ---- range variant -------------------------------------------------------------------------------
@@ -597,8 +412,12 @@ __global__ __launch_bounds__(kBlock) void scan_ranges_kernel(const In *__restric
   Acc excl = (red[0] + red[1]) + (red[2] + red[3]);
   if (MODE == kPrefixed) excl = Bits<Acc>::from(reinterpret_cast<const uint64_t *>(slots)[tile]);
   // Three passes cannot fail (the second one reads what this workgroup published itself); should
-  // they, the result is marked rather than silently wrong.
-  if (CHAINED && failed) excl = Bits<Acc>::from(0x7ff8dead00000000ull);
+  // they -- two launches that share one workspace at the same time --, the range is marked rather
+  // than silently wrong: NaN for the fp64 sums, the most negative integer for int64 ones (the
+  // prefixes of that range then come out negative where the inputs are not).
+  if (CHAINED && failed)
+    excl = Bits<Acc>::from(std::is_same<Acc, double>::value ? 0x7ff8dead00000000ull
+                                                            : 0x8000000000000000ull);
   const Acc wavebase = wave == 0 ? (Acc)0 : wave == 1 ? w0 : wave == 2 ? w0 + w1 : (w0 + w1) + w2;
   Acc run = (excl + wavebase) + wexcl;
 
@@ -703,11 +522,10 @@ __global__ __launch_bounds__(kBlock) void sum_final_kernel(const double *partial
 
 int64_t scan_tiles(int64_t n, int tile_elems) { return n <= 0 ? 0 : ceil_div64(n, tile_elems); }
 
-// Workspace: 256-byte header (the look-back kernel's ticket), then per smallest range (2048
-// elements, so that both element types fit) one 8-byte plain sum and one 24-byte tagged slot.
-// The look-back kernel lays its two words per 4096-element tile over the same bytes.
+// Workspace: a 256-byte header (unused), then per smallest range (2048 elements, so that both
+// element types fit) one 8-byte plain sum and one 24-byte tagged slot.
 size_t scan_ws_bytes(int64_t n) {
-  const int64_t tiles = scan_tiles(n, kRows * kBlock * 2);
+  const int64_t tiles = scan_tiles(n, kMinRange);
   return kHeaderBytes + align_up((size_t)tiles * (8 + sizeof(Slot)), 256);
 }
 
@@ -765,7 +583,7 @@ int launch_ranges(const In *in, Out *out, int64_t n, void *ws, hipStream_t st, b
                   int64_t first_changed) {
   const int64_t range_elems = (int64_t)G * kBlock * VE;
   const int64_t ranges = ceil_div64(n, range_elems);
-  const int64_t max_ranges = scan_tiles(n, kRows * kBlock * 2);
+  const int64_t max_ranges = scan_tiles(n, kMinRange);
   uint64_t *sums = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
   Slot *slots = reinterpret_cast<Slot *>(sums + max_ranges);
   const int64_t first = first_changed > 0 ? first_changed / range_elems : 0;
@@ -814,12 +632,10 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
   if ((reinterpret_cast<uintptr_t>(in) & (sizeof(In) - 1)) ||
       (reinterpret_cast<uintptr_t>(out) & 15))
     return GEAR_HIP_EALIGN;
-  // GEAR_HIP_SCAN_SINGLE_PASS: 1 = the chained kernel wherever it applies, 0 = never, 2 = the
-  // ticketed look-back kernel at every size (fp64 sums only; kept for comparisons); unset = the
+  // GEAR_HIP_SCAN_SINGLE_PASS: 1 = the chained kernel wherever it applies, 0 = never; unset = the
   // chained kernel for full scans, two launches for the rescan of a suffix.  A launch that is
   // being captured into a graph would replay its tag, so it takes the two launches.
   const int forced = env_int("GEAR_HIP_SCAN_SINGLE_PASS", -1);
-  const bool lookback = forced == 2 && std::is_same<Acc, double>::value && first_changed <= 0;
   bool chained = forced < 0 ? first_changed <= 0 : forced == 1;
   if (chained) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
@@ -837,32 +653,13 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
   // ranges.  (8-byte elements: ranges of 2 granules would be smaller than the 2048 elements the
   // workspace is laid out for, so they start at 4.)
   constexpr int64_t g1 = (int64_t)kBlock * VE;  // elements per range and granule
-  if (lookback) {
-    // fall through to the look-back launch below
-  } else if (VE == 4 && ceil_div64(n, 2 * g1) <= 256)
+  if (VE == 4 && ceil_div64(n, 2 * g1) <= 256)
     return launch_ranges<In, Acc, Out, VE, 2>(in, out, n, ws, st, chained, first_changed);
   else if (ceil_div64(n, 4 * g1) <= 512)
     return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, chained, first_changed);
   else if (ceil_div64(n, 8 * g1) <= kMaxRanges)
     return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, chained, first_changed);
-  else
-    return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, false, first_changed);
-  // (The look-back kernel marks "not published yet" with the word kEmpty, which no fp64 sum of
-  // fp32 values can equal but an int64 sum can (-1): fp64 sums only.  Its sums depend on which
-  // predecessors had published what when a workgroup looked: two runs can differ in the last
-  // bit, which is why it is not used unless asked for.)
-  const int64_t tiles = scan_tiles(n, kRows * kBlock * VE);
-  uint32_t *ticket = static_cast<uint32_t *>(ws);
-  uint64_t *aggr = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + kHeaderBytes);
-  uint64_t *incl = aggr + tiles;
-  const int64_t words = 2 * tiles;
-  scan_init_kernel<<<dim3((unsigned)ceil_div64(words, kBlock)), dim3(kBlock), 0, st>>>(ticket, aggr,
-                                                                                     words);
-  GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  scan_kernel<In, Acc, Out, VE><<<dim3((unsigned)tiles), dim3(kBlock), 0, st>>>(in, out, n, ticket,
-                                                                              aggr, incl);
-  GEARHIP_RETURN_IF_LAUNCH_FAILED();
-  return 0;
+  return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, false, first_changed);
 }
 
 }  // namespace
@@ -889,19 +686,37 @@ namespace {
 
 constexpr int64_t kStaticMaxN = 1ll << 27;  // 134 217 728 priorities
 constexpr size_t kStaticBytes =
-    kHeaderBytes + (size_t)(kStaticMaxN / (kRows * kBlock * 2)) * (8 + sizeof(Slot));
+    kHeaderBytes + (size_t)(kStaticMaxN / (kMinRange)) * (8 + sizeof(Slot));
 static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticBytes];
 
 constexpr int kMaxDevices = 64;
 std::atomic<void *> g_scratch_ptr[kMaxDevices];
 
-// Device address of `scratch` on the current device, looked up once per device.
-int static_scratch(void **ptr) {
-  int dev = -1;
-  GEARHIP_CHECK(hipGetDevice(&dev));
-  if (dev < 0 || dev >= kMaxDevices) return GEAR_HIP_ERANGE;
+// One static call at a time per device: calls that overlapped (two streams, two host threads)
+// would overwrite each other's range sums.  The event marks the end of the last static call's
+// kernels on its stream; the next call's stream waits for it before its own kernels start.
+struct StaticOrder {
+  std::mutex lock;
+  hipEvent_t done = nullptr;
+  bool recorded = false;
+};
+StaticOrder g_static_order[kMaxDevices];
+
+bool stream_is_capturing(hipStream_t st) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &cap) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;  // unknown: treat as capturing, the careful side
+  }
+  return cap != hipStreamCaptureStatusNone;
+}
+
+// Device address of `scratch` on device `dev` (the current one), looked up once per device.
+// may_look_up = false (the stream is being captured): only an address found earlier is returned.
+int static_scratch(int dev, bool may_look_up, void **ptr) {
   void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if (p == nullptr) {
+    if (!may_look_up) return GEAR_HIP_ENOTREADY;
     GEARHIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     if (p == nullptr) return (int)hipErrorInvalidSymbol;
     g_scratch_ptr[dev].store(p, std::memory_order_release);  // every thread finds the same address
@@ -910,11 +725,28 @@ int static_scratch(void **ptr) {
   return 0;
 }
 
+int current_device(int *dev) {
+  GEARHIP_CHECK(hipGetDevice(dev));
+  if (*dev < 0 || *dev >= kMaxDevices) return GEAR_HIP_ERANGE;
+  return 0;
+}
+
 }  // namespace
 
+// Set-up for the static form on the current device: the array's address and the event that
+// orders its calls.  What fails here is reported again by the entry point itself.
 int scan_static_init() {
+  int dev = -1;
+  int rc = current_device(&dev);
+  if (rc) return rc;
   void *p = nullptr;
-  return static_scratch(&p);
+  rc = static_scratch(dev, true, &p);
+  if (rc) return rc;
+  StaticOrder &order = g_static_order[dev];
+  std::lock_guard<std::mutex> guard(order.lock);
+  if (order.done == nullptr)
+    GEARHIP_CHECK(hipEventCreateWithFlags(&order.done, hipEventDisableTiming));
+  return 0;
 }
 
 }  // namespace gearhip
@@ -926,12 +758,28 @@ extern "C" int gear_hip_scan_f32_f64_static(const float *in, double *out, int64_
   if (n < 0) return GEAR_HIP_EINVAL;
   if (n > kStaticMaxN) return GEAR_HIP_ERANGE;
   if (n == 0) return 0;
-  void *ws = nullptr;
-  const int rc = static_scratch(&ws);
-  if (rc) return rc;
   static_assert(kStaticBytes >= kHeaderBytes + 16, "scratch holds at least one range");
   if (kStaticBytes < scan_ws_bytes(n)) return GEAR_HIP_ERANGE;
-  return launch_scan<float, double, double, 4>(in, out, n, ws, kStaticBytes, as_stream(stream));
+  int dev = -1;
+  int rc = current_device(&dev);
+  if (rc) return rc;
+  hipStream_t st = as_stream(stream);
+  const bool capturing = stream_is_capturing(st);
+  void *ws = nullptr;
+  rc = static_scratch(dev, !capturing, &ws);
+  if (rc) return rc;
+  if (capturing)  // the graph's own order is the caller's; events of this kind are not captured
+    return launch_scan<float, double, double, 4>(in, out, n, ws, kStaticBytes, st);
+  StaticOrder &order = g_static_order[dev];
+  std::lock_guard<std::mutex> guard(order.lock);
+  if (order.done == nullptr)
+    GEARHIP_CHECK(hipEventCreateWithFlags(&order.done, hipEventDisableTiming));
+  if (order.recorded) GEARHIP_CHECK(hipStreamWaitEvent(st, order.done, 0));
+  rc = launch_scan<float, double, double, 4>(in, out, n, ws, kStaticBytes, st);
+  if (rc) return rc;
+  GEARHIP_CHECK(hipEventRecord(order.done, st));
+  order.recorded = true;
+  return 0;
 }
 
 extern "C" int gear_hip_rescan_f32_f64(const float *in, double *out, int64_t n,

@@ -26,16 +26,16 @@ from ..utils import get_local_node_hashed_int32
 
 class BasicLoader:
     """Interface of every loader (gear/loader/basic_loader.py:4-14): a batch size, iteration,
-    and a checkpoint hook that subclasses may provide."""
+    and a checkpoint hook.  As there, the two hooks of the base do nothing and return None."""
 
     def __init__(self, batch_size) -> None:
         self._batch_size = batch_size
 
     def __next__(self):
-        raise NotImplementedError
+        return None
 
     def checkpoint(self):
-        raise NotImplementedError
+        return None
 
 
 def ensure_dataset(dataset):

@@ -34,6 +34,7 @@ extern "C" {
 #define GEAR_HIP_EWORKSPACE (-2)  /* workspace pointer null or smaller than the *_bytes query */
 #define GEAR_HIP_ERANGE (-3)      /* a size exceeds what the kernels index (see each call)    */
 #define GEAR_HIP_EALIGN (-4)      /* a pointer that must be naturally aligned is not          */
+#define GEAR_HIP_ENOTREADY (-5)   /* one-time set-up is missing and cannot run now (see call)  */
 
 /* ---- runtime ------------------------------------------------------------------------------ */
 
@@ -189,6 +190,10 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
  * workspace: device memory of at least gear_hip_scan_workspace_bytes(n) bytes, 256-byte aligned;
  * its contents need not be initialised (the call initialises it on `stream`).
  * n may be 0 (nothing is written).  n <= 2^40.  `out` must be 16-byte aligned.
+ * One workspace serves one call at a time.  Two one-pass calls that share a workspace while both
+ * run cannot hang (the wait is bounded) but may find each other's words; a range that could not
+ * be completed is marked: its prefixes are NaN (fp64 / fp32 results) or start from INT64_MIN
+ * (gear_hip_scan_i64: negative results where the inputs are not).
  * Rounding: inside a range (2048, 4096 or 8192 elements, by n) the prefix is a running sum of a
  * fixed association; the offset of a range is the separately rounded sum of all earlier ranges.
  * Both are within 1e-12 (relative) of the sequential fp64 sum, but they are rounded differently,
@@ -206,8 +211,13 @@ int gear_hip_scan_f32_f64(const float *in, double *out, int64_t n, void *workspa
  * the call allocates and frees nothing.  Same result, bit for bit, as gear_hip_scan_f32_f64.
  * n <= gear_hip_scan_static_max_n() (2^27 = 134 217 728), else GEAR_HIP_ERANGE.
  * The array's address is looked up once per device, by gear_hip_set_device or by the first call
- * on that device.  All calls on one GPU share the array: calls that overlap on one GPU (two
- * streams, two threads) race; serialise them or use the workspace form. */
+ * on that device; a first call on a stream that is being captured cannot look it up and returns
+ * GEAR_HIP_ENOTREADY (call gear_hip_set_device, or once outside the capture, first).
+ * All calls on one GPU share the array.  Outside graph capture the library orders them itself:
+ * a call's kernels wait (on the device, through an event) for the kernels of the previous static
+ * call on that GPU, whatever stream or host thread that one came from.  Captured calls are not
+ * ordered by the library: graphs that hold one must not run at the same time as another static
+ * call on that GPU, or the two race on the array; use the workspace form there. */
 int64_t gear_hip_scan_static_max_n(void);
 int gear_hip_scan_f32_f64_static(const float *in, double *out, int64_t n, void *stream);
 

@@ -1,5 +1,5 @@
 """GPU parity of the weighted sampler: fp64 prefix sum (the chained, two-launch and three-launch
-forms of the range scan and the tiled look-back scan kept for comparisons), batched upper_bound
+forms of the range scan), batched upper_bound
 search, importance weights, through the C ABI against the CPU oracle."""
 import os
 

@@ -57,6 +57,29 @@ def test_topk_cases(oracle):
     _check_topk(oracle, ops, ln(2_000_000), 2_500, "same size, spread out (lists)")
 
 
+def test_topk_without_the_sampled_hint(oracle):
+    """GEAR_HIP_TOPK_HINT=0 (read at every call): uniform level-0 bins, no candidate lists for
+    long inputs -- every level streams the priorities.  Same results."""
+    import os
+    from gear_amd import ops
+    rng = np.random.default_rng(32)
+    ln = lambda n: (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    old = os.environ.get("GEAR_HIP_TOPK_HINT")
+    os.environ["GEAR_HIP_TOPK_HINT"] = "0"
+    try:
+        _check_topk(oracle, ops, ln(3_000_000), 65_536, "no hint, lognormal")
+        _check_topk(oracle, ops, ln(3_000_000), 1, "no hint, k = 1")
+        _check_topk(oracle, ops, rng.integers(0, 50, size=2_000_000).astype(np.float32), 100_000,
+                    "no hint, ties")
+        _check_topk(oracle, ops, rng.normal(size=1_500_000).astype(np.float32), 140_000,
+                    "no hint, signed, radix-sorted output")
+    finally:
+        if old is None:
+            os.environ.pop("GEAR_HIP_TOPK_HINT", None)
+        else:
+            os.environ["GEAR_HIP_TOPK_HINT"] = old
+
+
 def test_topk_infinite_priorities(oracle):
     """The k-th largest priority is +inf (at least k of them), or the selection reaches down to
     -inf (k == n): the bins of the infinities border on keys that decode to NaN."""

@@ -333,6 +333,10 @@ def test_loader_partition_and_rank_order_on_one_rank():
     loader = OfflineLoader(ds, 3, ModelParallelismUnit(device="cpu"), "Uniform",
                            [{"name": "obs", "offset": 0, "length": 4}])
     assert isinstance(loader, BasicLoader)
+    # the base hooks are no-ops as in gear/loader/basic_loader.py:8-14, and OfflineLoader does
+    # not override checkpoint: it returns None instead of raising
+    assert loader.checkpoint() is None
+    assert BasicLoader(3).__next__() is None
     parts = loader.partition_indices(torch.tensor([0, 5, 2, 9, -1, 3]))
     assert len(parts) == 1 and len(parts[0]) == 1
     assert parts[0][0].tolist() == [0, 5, 2, 3]
@@ -340,3 +344,10 @@ def test_loader_partition_and_rank_order_on_one_rank():
     gear_amd.install_as_gear()
     from gear.loader.basic_loader import BasicLoader as B2
     assert B2 is BasicLoader
+    # the spelling the loader documents, "Topk" (gear/loader/offline_loader.py:44,61), finds the
+    # top-k sampler through the "<method>Sampler" look-up (:102-104)
+    import gear.sampler
+    assert gear.sampler.TopkSampler is gear.sampler.TopKSampler
+    topk_loader = OfflineLoader(ds, 3, ModelParallelismUnit(device="cpu"), "Topk",
+                                [{"name": "obs", "offset": 0, "length": 4}])
+    assert isinstance(topk_loader._sampler, gear.sampler.TopKSampler)

@@ -50,10 +50,12 @@ def test_static_scan_equals_workspace_scan_on_consecutive_calls(oracle):
         host = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
         pri = torch.from_numpy(host).cuda()
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        # free device memory as the driver reports it (hipMemGetInfo): a hipMalloc or hipFree
+        # inside the library would show here, torch's own allocator statistics would not
+        free_before = torch.cuda.mem_get_info()[0]
         got = _scan_static(lib, pri, outs[n])
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == free_before
         exp = _scan_workspace(lib, pri)
         torch.cuda.synchronize()
         assert torch.equal(got, exp), n
@@ -66,6 +68,28 @@ def test_static_scan_equals_workspace_scan_on_consecutive_calls(oracle):
     got = _scan_static(lib, pri, torch.empty(host.size, dtype=torch.float64, device="cuda"))
     torch.cuda.synchronize()
     assert np.array_equal(got.cpu().numpy(), oracle.scan_f32_f64(host))
+
+
+def test_static_scans_from_two_streams_are_ordered_by_the_library():
+    """Two streams issue static scans one right after the other, with nothing between them but
+    the library's own event: the second call's kernels wait for the first call's, so neither
+    finds the other's range sums in the shared array."""
+    lib = _cabi.load()
+    assert lib.gear_hip_set_device(0) == 0
+    rng = np.random.default_rng(78)
+    hosts = [(rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+             for n in (9_000_001, 2_500_000, 6_000_000, 300_000)]
+    pris = [torch.from_numpy(h).cuda() for h in hosts]
+    outs = [torch.empty(h.size, dtype=torch.float64, device="cuda") for h in hosts]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    announce("static scans alternating between two streams")
+    for i, (pri, out) in enumerate(zip(pris, outs)):
+        st = ctypes.c_void_p(streams[i % 2].cuda_stream)
+        assert lib.gear_hip_scan_f32_f64_static(_p(pri), _p(out), pri.numel(), st) == 0
+    torch.cuda.synchronize()
+    for pri, out in zip(pris, outs):
+        assert torch.equal(out, _scan_workspace(lib, pri)), pri.numel()
 
 
 def test_static_scan_rejects_what_it_cannot_hold():
