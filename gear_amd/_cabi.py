@@ -81,6 +81,8 @@ SIGNATURES = {
     "gear_hip_topk_workspace_bytes": (c_size_t, [c_i64, c_i64]),
     "gear_hip_topk_f32": (c_int, [c_void_p, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p,
                                   c_size_t, c_void_p]),
+    "gear_hip_topk_f32_warm": (c_int, [c_void_p, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p,
+                                       c_size_t, c_void_p]),
     "gear_hip_scatter_workspace_bytes": (c_size_t, [c_i64]),
     "gear_hip_scatter_f32": (c_int, [c_void_p, c_i64, c_void_p, c_void_p, c_i64, c_int, c_void_p,
                                      c_size_t, c_void_p]),

@@ -5,8 +5,10 @@
 //   prep      one workgroup draws 2048 to 32768 samples and lays out the level-0 bins around them (coarse
 //             below the bin that safely lies under the k-th largest priority -- the hint --, fine
 //             from there to the largest sample, the rest above); the others clear the histograms.
-//   level 0   ONE read of the priorities: level-0 histogram (LDS, flushed with atomics) and, per
-//             wave, a list of every candidate (key | index) at or above the hint, in index order.
+//   level 0   ONE read of the priorities: per wave a list of every candidate (key | index) at or
+//             above the hint, in index order, and the level-0 histogram of the candidates (the
+//             entries below the hint cost one compare each and are not counted).  Without a
+//             hint every entry is counted (and listed, when the lists hold whole ranges).
 //   level 1   picks the level-0 bin that holds the k-th largest key; histogram of the top bits
 //             inside that bin over its members;   level 2   the same for the remaining bits.
 //   count     picks the last digit: threshold key T and the number of entries equal to T still
@@ -17,9 +19,14 @@
 // Levels 1, 2, count and write walk the candidate lists (about 2 % of the input) when the hint
 // held; a wave whose list overflowed (clustered maxima, masses of equal priorities) reads its own
 // range of the priorities again instead, in each of them (count then rebuilds its list with the
-// exact threshold, write re-reads if that overflows too).  When the hint did not hold (fewer
-// than k candidates: the picked bin lies below it) every wave does.  The hint only decides
-// which of the two it is, never the result.
+// exact threshold, write re-reads if that overflows too).
+// When the hint fails (fewer than k candidates: the k-th largest priority lies below it; only a
+// sample that misleads does that) the entries below the hint -- which level 0 does not even
+// count, that is what makes it fast -- are searched by the same launches in another way: level 1
+// and level 2 stream the priorities and count the upper and the lower 16 bits of the keys below
+// the hint (65536-bin histograms, 16-bit counters packed in LDS and flushed before they can
+// overflow), count picks the threshold from the second one and streams as for an overflowed
+// list.  The hint only decides which way it is, never the result.
 // Value order (k <= 131072): write leaves the selection as (key, index, segment) in index order
 // and puts the entries equal to T straight at the tail of the output; the level-0 histogram says
 // where every bin starts in value order, bins that start in the same stretch of output places
@@ -42,6 +49,7 @@ constexpr int kWavesPerBlock = kThreads / kWave;
 constexpr int kMaxBlocks = 256;              // one workgroup per CU
 constexpr int kBins0 = 16384;  // level-0 bins
 constexpr int kBinsR = 2048;   // bins of a refinement level (up to 11 bits)
+constexpr int kBinsF = 65536;  // bins of the two levels that run after a failed hint (16 bits)
 constexpr int kUniformShift = 18;  // level-0 bins without a sample: the top 14 bits of the key
 // with a sample: keys below the hint at 12 bits, a middle stretch up to the sample's top in up to
 // kMidBins bins of its own resolution, the rest above
@@ -97,16 +105,78 @@ __device__ __forceinline__ uint32_t bin_hi_key(const BinMap &m, uint32_t bin) {
   return bin_lo_key(m, bin + 1u) - 1u;
 }
 
+// The map around a hint: keys below a_end (a multiple of 2^kLowShift) in coarse bins, the stretch
+// a_end .. b_last in up to mid_bins bins of its own resolution, the keys above with what is left
+// of the kBins0 bins.  A bin never spans more than 2^kMaxBinBits keys -- the two levels below
+// resolve 11 and 10 bits --: a middle stretch too wide for mid_bins bins of that size gets more
+// of them, at most 2048, which the budget of kMidBins covers.
+// compact: the stretch above b_last is cut as coarsely as the levels below allow, so that the
+// bins from the hint upwards are few (at most 2050) and their histogram can be kept in several
+// copies (see Copies).
+__device__ __forceinline__ BinMap make_map(uint32_t a_end, uint32_t b_last, int mid_bins,
+                                           bool compact) {
+  BinMap map;
+  map.uniform = 0u;
+  map.a_end = a_end;
+  map.b_last = b_last < a_end ? a_end : b_last;
+  map.b_shift = map.c_shift = 0u;
+  const uint32_t span = map.b_last - map.a_end;
+  while (map.b_shift < (uint32_t)kMaxBinBits && (span >> map.b_shift) >= (uint32_t)mid_bins)
+    ++map.b_shift;
+  map.nb0 = map.a_end >> kLowShift;
+  map.nc0 = map.nb0 + (span >> map.b_shift) + 1u;
+  const uint32_t rest = 0xffffffffu - map.b_last;  // keys above the middle stretch
+  while (rest != 0u && map.nc0 + ((rest - 1u) >> map.c_shift) >= (uint32_t)kBins0) ++map.c_shift;
+  if (compact && rest != 0u) map.c_shift = (uint32_t)kMaxBinBits;
+  return map;
+}
+
+// The level-0 histogram of the candidates in several copies.  Every workgroup of level 0 adds
+// its counts to the histogram in memory at the end, all of them at about the same time and to
+// the same few cache lines, and atomics on one line are served one after the other (about 16 ns
+// apiece: 245 workgroups, 4 us).  Where the places in value order of the bins are not asked for
+// (the index-ordered selection, large k) the bins from the hint upwards are few -- a compact
+// map --, the histogram is kept in 8 copies (4 when it has more than 2048 bins), workgroup b adds
+// to copy b mod 8, and level 1 adds the copies up when it picks: 3 us less for level 0.
+struct Copies {
+  uint32_t used;    // bins from the hint upwards: bin b is counted at b - nb0
+  uint32_t copies;  // 8 or 4
+  uint32_t pitch;   // words from one copy to the next
+};
+__device__ __forceinline__ Copies copies_of(const BinMap &m) {
+  Copies c;
+  const uint32_t rest = 0xffffffffu - m.b_last;
+  c.used = (m.nc0 - m.nb0) + (rest != 0u ? ((rest - 1u) >> m.c_shift) + 1u : 0u);
+  c.copies = c.used <= (uint32_t)kBins0 / 8u ? 8u : 4u;
+  c.pitch = (uint32_t)kBins0 / c.copies;
+  return c;
+}
+
+// The mark a call leaves with the hint for the next one: the hint is taken up again only by a
+// call of the same shape (and never from a workspace that holds anything else).
+__host__ __device__ __forceinline__ uint64_t next_mark(int64_t n, int64_t k, int mid_bins) {
+  uint64_t x = 0x9e3779b97f4a7c15ull ^ (uint64_t)n;
+  x = (x ^ (x >> 31)) * 0xbf58476d1ce4e5b9ull + (uint64_t)k;
+  x = (x ^ (x >> 29)) * 0x94d049bb133111ebull + (uint64_t)mid_bins;
+  x ^= x >> 32;
+  return x | 1ull;  // never zero: zero says "no hint"
+}
+
 struct State {
   uint32_t prefix[3];  // level-0 bin, level-1 digit, threshold key
   uint32_t k_rem[3];   // entries still to take from the bin picked at that level
   uint32_t overflow;   // no lists were asked for: every level reads the priorities
-  uint32_t overflow2;  // (unused)
+  uint32_t fail;       // the hint was too high (fewer than k candidates): see "when the hint fails"
   uint32_t hint_bin;   // candidates are the entries whose level-0 bin is >= this
   uint32_t full;       // levels 1, 2, count stream the priorities instead of the lists
   uint32_t lo0, hi0;   // smallest and largest key of the picked level-0 bin
   BinMap map;
-  uint32_t pad[45];
+  // what the next call may start from instead of a sample (the warm form): the bound below which
+  // nothing is listed and the largest key of the finely cut stretch, valid when next_magic holds
+  // the mark of a call with the same n, k and bin resolution
+  uint64_t next_magic;
+  uint32_t next_a_end, next_b_last;
+  uint32_t pad[40];
 };
 static_assert(sizeof(State) == 256, "State is the 256-byte header of the workspace");
 
@@ -165,7 +235,7 @@ Geom geom(int64_t n, int64_t k) {
 }
 
 struct Layout {
-  size_t hist0, hist1, hist2, wg_bins, boff, wave_listed, wave_ge, block_ge, lists, cidx,
+  size_t hist0, hist1, hist2, wg_bins, histf1, histf2, boff, wave_listed, wave_ge, block_ge, lists, cidx,
       cand, cand2, cseg, ckey, skey, sidx, tkey, tidx, shist, zero_begin, zero_end, total;
 };
 
@@ -179,6 +249,8 @@ Layout layout(int64_t n, int64_t k) {
   l.hist1 = o;  o += kBinsR * sizeof(uint32_t);
   l.hist2 = o;  o += kBinsR * sizeof(uint32_t);
   l.wg_bins = o; o += 4 * kMaxBlocks * sizeof(uint32_t);
+  l.histf1 = o; o += kBinsF * sizeof(uint32_t);  // after a failed hint: upper / lower 16 key bits
+  l.histf2 = o; o += kBinsF * sizeof(uint32_t);
   l.zero_end = o;
   l.boff = o;   o += kBins0 * sizeof(uint32_t);
   l.wave_listed = o; o += (size_t)kMaxBlocks * kWavesPerBlock * sizeof(uint32_t);
@@ -214,10 +286,11 @@ Layout layout(int64_t n, int64_t k) {
 // highest bin + 1, BINS - lowest bin, ~(entries above the segment), entries above it + its own;
 // 0 = none; zeroed by the caller): the workgroups of the launch share
 // that work, every one of them has to call with the same arguments.
-// With no such bin (only possible with NaN priorities, which the float compares of the later
-// levels do not count) the lowest bin is returned and nothing is taken off k_rem.
+// With no such bin (the histogram holds fewer than k_rem entries: the candidates of a hint that
+// was too high, or NaN priorities, which nothing counts) the lowest bin is returned, nothing is
+// taken off k_rem and `found` is 0; `total` is the number of entries in the histogram.
 struct Pick {
-  uint32_t bin, k_rem;
+  uint32_t bin, k_rem, found, total;
 };
 template <int BINS>
 __device__ __forceinline__ Pick pick_bin(uint32_t k_rem, const uint32_t *hist, uint32_t *boff,
@@ -260,6 +333,7 @@ __device__ __forceinline__ Pick pick_bin(uint32_t k_rem, const uint32_t *hist, u
   if (tid == 0) {
     s_pick.bin = 0u;
     s_pick.k_rem = k_rem;
+    s_pick.found = 0u;
     s_bin2 = 0u;
   }
   __syncthreads();
@@ -286,11 +360,15 @@ __device__ __forceinline__ Pick pick_bin(uint32_t k_rem, const uint32_t *hist, u
         r += c[j];
       }
       *bin_out = pb;
-      if (rem_out) *rem_out = pk;
+      if (rem_out) {
+        *rem_out = pk;
+        s_pick.found = 1u;
+      }
     }
   };
   find(k_rem, &s_pick.bin, &s_pick.k_rem);
   if (rank2 != 0u) find(rank2, &s_bin2, nullptr);
+  if (tid == kActive - 1) s_pick.total = running0 + (uint32_t)tsum;
   if (boff && (tid * kPerThread) % kWave == 0 && active) s_base[tid * kPerThread / kWave] = running0;
   __syncthreads();
   // Where the bins at or above the picked one start in value order (the entries above them),
@@ -491,13 +569,15 @@ __device__ __forceinline__ void list_append(uint64_t *list, int list_cap, int &l
 // share of k, so that the k-th largest priority of the whole input lies in the fine stretch
 // unless the sample misleads -- which costs time (the later levels stream the input again),
 // never correctness.  rank = 0: no sample, uniform bins; every entry is listed when list_all is
-// set (the lists are as long as the waves' ranges), none otherwise.  The other workgroups
-// clear the histograms.
+// set (the lists are as long as the waves' ranges), none otherwise.
+// warm != 0: when the workspace holds the hint that the last call of the same shape left for this
+// one (the bound derived from its exact counts), the map is laid out around that and no sample
+// is drawn; otherwise as above.  The other workgroups clear the histograms.
 template <int kPer>  // samples per thread
 __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict__ p, int64_t n,
-                                                        uint32_t rank, int list_all, int mid_bins,
-                                                        State *state, uint32_t *zero,
-                                                        int64_t zero_words) {
+                                                        int64_t k, uint32_t rank, int list_all,
+                                                        int mid_bins, int warm, State *state,
+                                                        uint32_t *zero, int64_t zero_words) {
   __shared__ __align__(16) uint32_t h[kBins0];
   const int tid = threadIdx.x;
   if (blockIdx.x > 0) {
@@ -509,8 +589,23 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict_
     }
     return;
   }
+  // the hint of the last call, read by one thread before anything of the state is written
+  __shared__ uint32_t s_warm[3];
+  bool reuse = false;
+  uint32_t warm_a_end = 0u, warm_b_last = 0u;
+  if (warm && rank != 0u) {
+    if (tid == 0) {
+      s_warm[0] = state->next_magic == next_mark(n, k, mid_bins) ? 1u : 0u;
+      s_warm[1] = state->next_a_end & ~((1u << kLowShift) - 1u);
+      s_warm[2] = state->next_b_last;
+    }
+    __syncthreads();
+    reuse = s_warm[0] != 0u;
+    warm_a_end = s_warm[1];
+    warm_b_last = s_warm[2];
+  }
   float v[kPer];
-  if (rank != 0u) {
+  if (rank != 0u && !reuse) {
     const int64_t stride = n / (kPer * kThreads);  // >= 128 (the caller's condition), < 2^20
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
@@ -521,14 +616,18 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict_
   }
   if (tid < 3) state->prefix[tid] = 0u;
   if (tid >= 3 && tid < 6) state->k_rem[tid - 3] = 0u;
-  if (tid == 6) state->overflow2 = 0u;
+  if (tid == 6) state->fail = 0u;
   if (tid == 7) state->full = 0u;
   if (tid == 8) state->overflow = (rank == 0u && !list_all) ? 1u : 0u;
+  if (tid == 9) state->next_magic = 0ull;  // level 1 of this call leaves the next hint, if any
   BinMap map;
   map.uniform = 1u;
   map.a_end = map.b_last = map.nb0 = map.nc0 = map.b_shift = map.c_shift = 0u;
   uint32_t hint = (rank == 0u && !list_all) ? kNoLists : 0u;
-  if (rank != 0u) {
+  if (rank != 0u && reuse) {
+    map = make_map(warm_a_end, warm_b_last, mid_bins, mid_bins == kMidBinsCoarse);
+    hint = map.nb0;
+  } else if (rank != 0u) {
     for (int i = tid; i < kBins0; i += kThreads) h[i] = 0u;
     __syncthreads();
 #pragma unroll
@@ -536,19 +635,9 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict_
     __syncthreads();
     uint32_t top14 = 0u;
     const uint32_t hint14 = pick_bin<kBins0>(rank, h, nullptr, nullptr, 0, 1u, &top14).bin;
-    map.uniform = 0u;
-    map.a_end = (hint14 << kUniformShift) & ~((1u << kLowShift) - 1u);
-    map.b_last = ((top14 + 1u) << kUniformShift) - 1u;  // wraps to the last key for the top bin
-    const uint32_t span = map.b_last - map.a_end;
-    // (a bin never spans more than 2^kMaxBinBits keys -- the two levels below resolve 11 bits
-    // each --: a middle stretch too wide for mid_bins bins of that size gets more of them, at most
-    // 2048, which the budget of kMidBins covers)
-    while (map.b_shift < (uint32_t)kMaxBinBits && (span >> map.b_shift) >= (uint32_t)mid_bins)
-      ++map.b_shift;
-    map.nb0 = map.a_end >> kLowShift;
-    map.nc0 = map.nb0 + (span >> map.b_shift) + 1u;
-    const uint32_t rest = 0xffffffffu - map.b_last;  // keys above the middle stretch
-    while (rest != 0u && map.nc0 + ((rest - 1u) >> map.c_shift) >= (uint32_t)kBins0) ++map.c_shift;
+    // (the last key of the top bin: the shift wraps to 0 there)
+    map = make_map((hint14 << kUniformShift) & ~((1u << kLowShift) - 1u),
+                   ((top14 + 1u) << kUniformShift) - 1u, mid_bins, mid_bins == kMidBinsCoarse);
     hint = map.nb0;  // the candidates: everything from the middle stretch upwards
   }
   if (tid == 0) {
@@ -562,23 +651,175 @@ __global__ __launch_bounds__(kThreads) void prep_kernel(const float *__restrict_
 __device__ __forceinline__ void count_add(uint32_t *cnt, uint32_t d, bool valid);
 
 // ---- level 0: ONE read of the priorities --------------------------------------------------------------
-// Every entry is counted in its level-0 bin (LDS histogram, flushed with atomics); the
-// candidates -- entries at or above the hint, about one in fifty -- are also listed per wave, in
-// index order, as key << 32 | index.  While streaming, a candidate is only dropped into the
-// wave's queue in LDS (value | index, at its place in index order: nearly every wave step holds
-// one or two candidates, so whatever is done per candidate there is paid per step); after the
-// stream the wave bins the candidates of its queue and writes the list, all lanes busy.  A
-// candidate that finds the queue full is binned at once and the wave's list is given up.
 constexpr int kQueueCap = 512;  // candidates per wave held in LDS; longer lists overflow
 
+// With a hint.  The loop over the priorities is bound by the instructions a CU can issue, not
+// by memory, so an entry below the hint -- forty-nine in fifty -- costs ONE compare and nothing
+// else: it is not counted anywhere (if the hint turns out too high, levels 1 and 2 look for
+// the threshold among those entries themselves, see the top of the file).  The candidates of a
+// step enter the wave's queue in LDS as value | index at their place in index order: the
+// compares of the wave leave four lane masks, the candidates of the lanes before a lane are four
+// masked bit counts.  After the stream the wave turns its queue into its list (key | index),
+// all lanes busy, and counts the candidates in the workgroup's level-0 histogram in LDS, noting
+// which runs of 64 bins it touched; once every wave is through, only those runs are added to the
+// histogram in memory (a sweep over all 16384 bins by every workgroup cost 4 us of a 16 us
+// launch).  A wave whose candidates outgrow the queue gives its list up (the later launches read
+// its range again) and counts the candidates of its range straight into the histogram.
+__device__ __forceinline__ uint32_t lanes_before(uint64_t mask, uint32_t acc) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                   __builtin_amdgcn_mbcnt_lo((uint32_t)mask, acc));
+}
+
+template <bool COMPACT>  // the histogram holds the bins from the hint upwards only, in copies
+__global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
+    const float *__restrict__ p, int64_t n, const State *state, uint32_t *__restrict__ hist0,
+    int64_t wave_len, uint32_t *__restrict__ wave_listed, uint64_t *__restrict__ lists,
+    int list_cap) {
+  __shared__ __align__(16) uint32_t h[kBins0];
+  __shared__ uint64_t queue[kWavesPerBlock][kQueueCap];
+  __shared__ uint32_t s_touched[kBins0 / kWave];  // runs of 64 bins that hold a count
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
+  const int64_t begin = gw * wave_len;
+  const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+  const int len = end > begin ? (int)(end - begin) : 0;  // (a wave's range is far below 2^31)
+  const int whole = len / kStep;  // steps of one float4 per lane that lie inside the range
+  const float *base = p + (len > 0 ? begin : 0);
+  // Loads of whole steps carry no test and no branch (a branch around a load makes the compiler
+  // wait for every load where the paths meet); a step beyond the last whole one is loaded from
+  // the last one's place and not looked at.
+  auto load_step = [&](int step, f4 &v) {
+    const int st = step < whole ? step : whole - 1;
+    v = *reinterpret_cast<const f4 *>(base + (int64_t)st * kStep + lane * 4);
+  };
+  // the first loads go out before the histogram is cleared
+  f4 qa[kAhead], qb[kAhead];
+  if (whole > 0) {
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) load_step(a, qa[a]);
+  }
+  for (int i = tid * 4; i < kBins0; i += kThreads * 4)
+    *reinterpret_cast<u32x4 *>(&h[i]) = u32x4{0u, 0u, 0u, 0u};
+  if (tid < kBins0 / kWave) s_touched[tid] = 0u;
+  const BinMap map = state->map;
+  const float lo_f = lower_bound_float(map.a_end);
+  const uint32_t bin_base = COMPACT ? map.nb0 : 0u;  // candidates' bins are counted from here
+  const uint32_t cap = (uint32_t)(list_cap < kQueueCap ? list_cap : kQueueCap);
+  const uint32_t first_index = (uint32_t)begin + (uint32_t)lane * 4u;
+  uint64_t *wq = queue[wave];
+  uint32_t queued = 0;    // candidates of the wave so far, all in the queue (the same in every lane)
+  bool given_up = false;  // ... until they outgrow it
+  __syncthreads();
+  // v: the lane's four entries of the step at offset s of the range
+  auto take = [&](int s, const f4 &v) {
+    const uint64_t m0 = wave_ballot(v[0] >= lo_f), m1 = wave_ballot(v[1] >= lo_f),
+                   m2 = wave_ballot(v[2] >= lo_f), m3 = wave_ballot(v[3] >= lo_f);
+    if ((m0 | m1 | m2 | m3) == 0ull) return;
+    // (wave-wide counts: said so, the branch on them is taken by the whole wave)
+    const uint32_t total = (uint32_t)__builtin_amdgcn_readfirstlane(
+        __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3));
+    if (queued + total > cap) {
+      given_up = true;
+      return;
+    }
+    uint32_t at = lanes_before(m3, lanes_before(m2, lanes_before(m1, lanes_before(m0, queued))));
+    const uint32_t i0 = first_index + (uint32_t)s;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (v[j] >= lo_f) {
+        wq[at] = ((uint64_t)__float_as_uint(v[j]) << 32) | (i0 + (uint32_t)j);
+        ++at;
+      }
+    }
+    queued = (uint32_t)__builtin_amdgcn_readfirstlane((int)(queued + total));
+  };
+  for (int st = 0; st < whole && !given_up;) {
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) load_step(st + kAhead + a, qb[a]);
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+      if (st + a < whole && !given_up) take((st + a) * kStep, qa[a]);
+    st += kAhead;
+    if (st >= whole || given_up) break;
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) load_step(st + kAhead + a, qa[a]);
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+      if (st + a < whole && !given_up) take((st + a) * kStep, qb[a]);
+    st += kAhead;
+  }
+  if (!given_up && whole * kStep < len) {
+    // the ragged end of the input, in the one wave that holds it; what lies beyond reads as
+    // NaN, which no compare takes for a candidate
+    f4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = whole * kStep + lane * 4 + j;
+      v[j] = e < len ? base[e] : __uint_as_float(0x7fc00000u);
+    }
+    take(whole * kStep, v);
+  }
+  if (given_up) {
+    // Masses of equal priorities or clustered maxima: more candidates than the queue holds.  The
+    // wave gives its list up and counts the candidates of its whole range straight into the
+    // histogram, lanes that share a bin by one atomic (the range is read again: it is in the
+    // caches, and the later launches read it again anyway).
+    queued = 0;
+    stream_range(p, begin, end, lane, [&](int64_t e0, const float q[4]) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool cand = e0 + j < end && q[j] >= lo_f;
+        if (wave_ballot(cand) == 0ull) continue;
+        const uint32_t bin = bin_of(map, order_key(q[j])) - bin_base;
+        count_add(h, bin, cand);
+        if (cand) s_touched[bin / kWave] = 1u;
+      }
+    });
+  }
+  // the queue, in index order, becomes the wave's list and is counted
+  uint64_t *list = lists + gw * list_cap;
+  for (uint32_t i = (uint32_t)lane; i < queued; i += kWave) {
+    const uint64_t ent = wq[i];
+    const uint32_t key = order_key(__uint_as_float((uint32_t)(ent >> 32)));
+    const uint32_t bin = bin_of(map, key) - bin_base;
+    atomicAdd(&h[bin], 1u);
+    s_touched[bin / kWave] = 1u;
+    list[i] = ((uint64_t)key << 32) | (uint32_t)ent;
+  }
+  // a wave whose list overflowed says so: the later launches read its range of the priorities
+  // again, its range only
+  if (lane == 0) wave_listed[gw] = given_up ? kListFull : queued;
+  __syncthreads();
+  // The counts go to memory by runs of 64 bins, a lane per bin, and only the runs that hold
+  // any: atomics of a wave that fall into one cache line travel as one request, and requests to
+  // a line are served one after the other -- candidates that each added their own bin's count
+  // sent some 50 000 requests to the eight lines of 256 coarse bins, 20 to 35 us.  Wave w looks
+  // after the runs w, w + 16, ...
+  static_assert(kBins0 / kWave == kWavesPerBlock * 16, "sixteen runs of bins per wave");
+  uint32_t *mine = hist0;
+  if (COMPACT) {
+    const Copies cp = copies_of(map);
+    mine += (blockIdx.x % cp.copies) * cp.pitch;
+  }
+  const uint32_t flag = lane < 16 ? s_touched[wave + kWavesPerBlock * lane] : 0u;
+  for (uint64_t todo = wave_ballot(flag != 0u); todo != 0ull; todo &= todo - 1ull) {
+    const int run = wave + kWavesPerBlock * (__ffsll((unsigned long long)todo) - 1);
+    const uint32_t c = h[run * kWave + lane];
+    if (c != 0u) atomicAdd(&mine[run * kWave + lane], c);
+  }
+}
+
+// Without a hint: every entry is counted in its level-0 bin (uniform bins of the top 14 key
+// bits; LDS histogram, flushed with atomics).  Short inputs, whose lists hold whole ranges, also
+// list every entry at its own place in the wave's range -- nothing to queue or order; otherwise
+// nothing is listed and the later levels stream the priorities.
 __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restrict__ p, int64_t n,
-                                                          State *state,
+                                                          const State *state,
                                                           uint32_t *__restrict__ hist0,
                                                           int64_t wave_len,
                                                           uint32_t *__restrict__ wave_listed,
                                                           uint64_t *__restrict__ lists, int list_cap) {
   __shared__ __align__(16) uint32_t h[kBins0];
-  __shared__ uint64_t queue[kWavesPerBlock][kQueueCap];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // the first loads of the wave's range go out before the histogram is cleared
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
@@ -587,133 +828,194 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
   float q0[kAhead][4];
   stream_first(p, begin, end, lane, q0);
   for (int i = tid; i < kBins0; i += kThreads) h[i] = 0u;
-  const uint32_t hint = state->hint_bin;
+  const bool whole_ranges = state->hint_bin != kNoLists;
   const BinMap map = state->map;
-  const bool want_lists = hint != kNoLists;
-  const float lo_f = lower_bound_float(
-      !want_lists ? kKeyPosInf : (map.uniform ? hint << kUniformShift : map.a_end));
-  // below the candidates every bin is key >> low_shift (the map's coarse stretch, or all bins
-  // of a uniform map)
-  const int low_shift = map.uniform ? kUniformShift : kLowShift;
-  const int cap = list_cap < kQueueCap ? list_cap : kQueueCap;
   __syncthreads();
   uint64_t *list = lists + gw * list_cap;
-  uint64_t *wq = queue[wave];
-  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  uint32_t nq = 0;  // candidates of the wave so far (wave-uniform)
-  // Lists that hold whole ranges with no hint (short inputs): every element is a candidate and
-  // its place in the wave's list is its place in the wave's range -- nothing to queue or order.
-  const bool whole_ranges = want_lists && hint == 0u && (int64_t)list_cap >= wave_len;
-  if (whole_ranges) {
-    stream_range_tagged(p, begin, end, lane, q0, [&](int64_t e0, const float q[4], auto whole) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (decltype(whole)::value || e0 + j < end) {
-          const uint32_t key = order_key(q[j]);
-          atomicAdd(&h[bin_of(map, key)], 1u);
-          list[e0 + j - begin] = ((uint64_t)key << 32) | (uint32_t)(e0 + j);
-        }
-      }
-    });
-    if (lane == 0) wave_listed[gw] = begin < end ? (uint32_t)(end - begin) : 0u;
-    __syncthreads();
-    for (int i = tid; i < kBins0; i += kThreads)
-      if (h[i]) atomicAdd(&hist0[i], h[i]);
-    return;
-  }
   stream_range_tagged(p, begin, end, lane, q0, [&](int64_t e0, const float q[4], auto whole) {
-    uint32_t rem = 0;  // bit j: element j of the lane is a candidate
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const bool valid = decltype(whole)::value || e0 + j < end;
-      const bool cand = want_lists && valid && q[j] >= lo_f;
-      rem |= cand ? 1u << j : 0u;
-      // everything else goes to its coarse bin right away
-      if (valid && !cand) atomicAdd(&h[order_key(q[j]) >> low_shift], 1u);
-    }
-    // The candidates of the step enter the queue in index order.  Mostly no lane holds more
-    // than one: the lanes' candidates, lanes in order, are in index order as they are.  Else a
-    // lane's place follows from the candidates of the lanes before it (up to four each: a
-    // ballot per bit of the count).  A candidate that finds the queue full is binned at once.
-    const uint64_t with = wave_ballot(rem != 0u);
-    if (with == 0ull) return;
-    if (wave_ballot((rem & (rem - 1u)) != 0u) == 0ull) {
-      bool over = false;
-      uint32_t over_bin = 0u;
-      if (rem != 0u) {
-        const int j = __ffs((int)rem) - 1;
-        const float x = j == 0 ? q[0] : (j == 1 ? q[1] : (j == 2 ? q[2] : q[3]));
-        const uint32_t at = nq + (uint32_t)__popcll(with & lt_mask);
-        if (at < (uint32_t)cap) {
-          wq[at] = ((uint64_t)__float_as_uint(x) << 32) | (uint32_t)(e0 + j);
-        } else {
-          over = true;
-          over_bin = bin_of(map, order_key(x));
-        }
-      }
-      nq += (uint32_t)__popcll(with);
-      if (nq > (uint32_t)cap) count_add(h, over_bin, over);
-    } else {
-      const int nc = __popc(rem);
-      const uint64_t b0 = wave_ballot((nc & 1) != 0), b1 = wave_ballot((nc & 2) != 0),
-                     b2 = wave_ballot((nc & 4) != 0);
-      uint32_t at = nq + (uint32_t)(__popcll(b0 & lt_mask) + 2 * __popcll(b1 & lt_mask) +
-                                    4 * __popcll(b2 & lt_mask));
-      nq += (uint32_t)(__popcll(b0) + 2 * __popcll(b1) + 4 * __popcll(b2));
-      const bool spills = nq > (uint32_t)cap;  // masses of equal priorities share a bin
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const bool c = ((rem >> j) & 1u) != 0u;
-        const bool over = c && at >= (uint32_t)cap;
-        if (c && !over) wq[at] = ((uint64_t)__float_as_uint(q[j]) << 32) | (uint32_t)(e0 + j);
-        if (spills) count_add(h, over ? bin_of(map, order_key(q[j])) : 0u, over);
-        at += c ? 1u : 0u;
+      if (decltype(whole)::value || e0 + j < end) {
+        const uint32_t key = order_key(q[j]);
+        atomicAdd(&h[bin_of(map, key)], 1u);
+        if (whole_ranges && e0 + j - begin < list_cap)
+          list[e0 + j - begin] = ((uint64_t)key << 32) | (uint32_t)(e0 + j);
       }
     }
   });
-  if (want_lists) {
-    // the wave's queue, in index order, is binned and becomes the wave's list, all lanes busy (an
-    // overflowed one is only binned: the later launches read the wave's range instead)
-    const uint32_t m_all = nq;
-    const uint32_t m = m_all < (uint32_t)cap ? m_all : (uint32_t)cap;
-    const bool given_up = m_all > (uint32_t)cap;
-    for (uint32_t i = lane; i < m; i += kWave) {
-      const uint64_t mine = wq[i];
-      const uint32_t key = order_key(__uint_as_float((uint32_t)(mine >> 32)));
-      if (given_up) {
-        count_add(h, bin_of(map, key), true);
-      } else {
-        atomicAdd(&h[bin_of(map, key)], 1u);
-        list[i] = ((uint64_t)key << 32) | (uint32_t)mine;
-      }
-    }
-    if (lane == 0) {
-      // a wave whose list overflowed (clustered maxima, masses of equal priorities) says so:
-      // the later launches read its range of the priorities again, its range only
-      wave_listed[gw] = m_all > (uint32_t)cap ? kListFull : m;
-    }
-  }
+  if (whole_ranges && lane == 0) wave_listed[gw] = begin < end ? (uint32_t)(end - begin) : 0u;
   __syncthreads();
   for (int i = tid; i < kBins0; i += kThreads)
     if (h[i]) atomicAdd(&hist0[i], h[i]);
 }
 
+// pick_bin for the level-0 histogram of a compact map (see Copies): the bins from the hint
+// upwards, at most 4096, kept in several copies that are added up here.  Returns the picked bin
+// under its number in the map.  Every thread of the workgroup calls.
+__device__ __forceinline__ Pick pick_copies(uint32_t k_rem, const uint32_t *hist, const BinMap &map,
+                                            uint32_t rank2, uint32_t *bin2) {
+  constexpr int kPer = 4;  // bins per thread, top down: thread 0 owns the top four
+  static_assert(kPer * kThreads * 4 == kBins0, "a copy of up to 4096 bins");
+  __shared__ uint32_t wsum[kWavesPerBlock];
+  __shared__ Pick s_pick;
+  __shared__ uint32_t s_bin2;
+  const Copies cp = copies_of(map);
+  const int tid = threadIdx.x, lane = tid & 63;
+  uint32_t c[kPer];
+  uint32_t tsum = 0u;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const uint32_t from_top = (uint32_t)(tid * kPer + j);
+    c[j] = 0u;
+    if (from_top < cp.used) {
+      const uint32_t at = cp.used - 1u - from_top;
+      for (uint32_t r = 0; r < cp.copies; ++r) c[j] += hist[r * cp.pitch + at];
+    }
+    tsum += c[j];
+  }
+  const int inc = wave_inclusive_sum((int)tsum);
+  if (lane == 63) wsum[tid >> 6] = (uint32_t)inc;
+  if (tid == 0) {
+    s_pick.bin = map.nb0;
+    s_pick.k_rem = k_rem;
+    s_pick.found = 0u;
+    s_bin2 = 0u;
+  }
+  __syncthreads();
+  const uint32_t before =
+      (uint32_t)wave_sum((int)(lane < (tid >> 6) && lane < kWavesPerBlock ? wsum[lane] : 0u));
+  const uint32_t running0 = before + (uint32_t)inc - tsum;  // entries above the thread's bins
+  auto find = [&](uint32_t rank, uint32_t *bin_out, uint32_t *rem_out) {
+    if (running0 < rank && running0 + tsum >= rank) {  // one thread
+      uint32_t r = running0, pb = 0u, pk = 0u;
+      bool found = false;
+#pragma unroll
+      for (int j = 0; j < kPer; ++j) {
+        const bool here = !found && r + c[j] >= rank;
+        pb = here ? map.nb0 + cp.used - 1u - (uint32_t)(tid * kPer + j) : pb;
+        pk = here ? rank - r : pk;
+        found = found || here;
+        r += c[j];
+      }
+      *bin_out = pb;
+      if (rem_out) {
+        *rem_out = pk;
+        s_pick.found = 1u;
+      }
+    }
+  };
+  find(k_rem, &s_pick.bin, &s_pick.k_rem);
+  if (rank2 != 0u) find(rank2, &s_bin2, nullptr);
+  if (tid == kThreads - 1) s_pick.total = running0 + tsum;
+  __syncthreads();
+  if (bin2) *bin2 = s_bin2;
+  return s_pick;
+}
+
+// ---- when the hint fails: 65536-bin histograms over the entries below it -----------------------------
+// pick_bin for a histogram of 65536 bins in memory: every thread of the workgroup calls.
+__device__ __forceinline__ Pick pick_wide(uint32_t rank, const uint32_t *hist) {
+  constexpr int kPer = kBinsF / kThreads;  // 64 bins per thread, thread 0 the top ones
+  __shared__ uint32_t wsum[kWavesPerBlock];
+  __shared__ Pick s_pick;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const uint32_t *mine = hist + kBinsF - (tid + 1) * kPer;
+  uint32_t tsum = 0u;
+#pragma unroll 4
+  for (int v = 0; v < kPer / 4; ++v) {
+    const u32x4 q = *reinterpret_cast<const u32x4 *>(mine + v * 4);
+    tsum += q[0] + q[1] + q[2] + q[3];
+  }
+  const int inc = wave_inclusive_sum((int)tsum);
+  if (lane == 63) wsum[tid >> 6] = (uint32_t)inc;
+  if (tid == 0) {
+    s_pick.bin = 0u;
+    s_pick.k_rem = rank;
+    s_pick.found = 0u;
+  }
+  __syncthreads();
+  const uint32_t before =
+      (uint32_t)wave_sum((int)(lane < (tid >> 6) && lane < kWavesPerBlock ? wsum[lane] : 0u));
+  const uint32_t running0 = before + (uint32_t)inc - tsum;  // entries above the thread's bins
+  if (running0 < rank && running0 + tsum >= rank) {  // one thread
+    uint32_t r = running0;
+    for (int j = kPer - 1; j >= 0; --j) {
+      const uint32_t c = mine[j];
+      if (r + c >= rank) {
+        s_pick.bin = (uint32_t)(kBinsF - (tid + 1) * kPer + j);
+        s_pick.k_rem = rank - r;
+        s_pick.found = 1u;
+        break;
+      }
+      r += c;
+    }
+  }
+  if (tid == kThreads - 1) s_pick.total = running0 + tsum;
+  __syncthreads();
+  return s_pick;
+}
+
+// Every wave streams its range and counts digit(q) for the entries that member(q) takes, in a
+// histogram of kBinsF 16-bit counters packed two to a word in LDS (hp, kBinsF / 2 words), which
+// the workgroup adds to hist_out in memory before a counter can overflow: after every 15 steps
+// of its 16 waves (61440 entries).  Called by every thread of the workgroup.
+constexpr int kFlushSteps = 15;
+static_assert(kFlushSteps * kStep * kWavesPerBlock < 65536, "a 16-bit counter holds a period's entries");
+template <typename F>
+__device__ __forceinline__ void wide_hist(const float *__restrict__ p, int64_t n, int64_t wave_len,
+                                          int64_t gw, uint32_t *hp, uint32_t *__restrict__ hist_out,
+                                          F digit_of) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  for (int i = tid; i < kBinsF / 2; i += kThreads) hp[i] = 0u;
+  __syncthreads();
+  const int64_t begin = gw * wave_len;
+  const int64_t end = begin + wave_len < n ? begin + wave_len : n;
+  // (the same number of periods in every wave of the workgroup: each ends at a barrier)
+  for (int64_t o = 0; o < wave_len; o += (int64_t)kFlushSteps * kStep) {
+    const int64_t a = begin + o;
+    const int64_t b = a + (int64_t)kFlushSteps * kStep < end ? a + (int64_t)kFlushSteps * kStep : end;
+    stream_range(p, a, b, lane, [&](int64_t e0, const float q[4]) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t d = 0u;
+        if (e0 + j < b && digit_of(q[j], &d)) atomicAdd(&hp[d >> 1], 1u << (16 * (d & 1u)));
+      }
+    });
+    __syncthreads();
+    for (int i = tid; i < kBinsF / 2; i += kThreads) {
+      const uint32_t w = hp[i];
+      if (w != 0u) {
+        if (w & 0xffffu) atomicAdd(&hist_out[2 * i], w & 0xffffu);
+        if (w >> 16) atomicAdd(&hist_out[2 * i + 1], w >> 16);
+        hp[i] = 0u;
+      }
+    }
+    __syncthreads();
+  }
+}
+
 // ---- levels 1 and 2: histograms inside the picked bin ------------------------------------------------
 // The keys of the picked level-0 bin are lo0 .. hi0; in `bits0` bits they can differ (at most 21).
-// LEVEL 1: picks the level-0 bin from hist0 (and decides whether the lists can be used: the hint
-// held when the picked bin is not below the hint bin); counts the top min(bits0, 11) of those
-// bits over the members of the bin.  LEVEL 2: picks the level-1 digit from hist1; counts the
-// remaining bits (at most 10) over the keys that share bin and digit.
+// LEVEL 1: picks the level-0 bin from hist0 (with a hint the histogram holds the candidates only:
+// when they are fewer than k the hint has failed); counts the top min(bits0, 11) of those bits
+// over the members of the bin; leaves the next call's hint.  LEVEL 2: picks the level-1 digit
+// from hist1; counts the remaining bits (at most 10) over the keys that share bin and digit.
+// After a failed hint: LEVEL 1 counts the upper 16 key bits of the entries below the hint
+// (histf1), LEVEL 2 picks from that and counts the lower 16 bits of the keys that share the
+// upper ones (histf2).
 __device__ __forceinline__ int bits_of(uint32_t span) { return span ? 32 - __builtin_clz(span) : 0; }
 __device__ __forceinline__ int level1_shift(int bits0) { return bits0 > 11 ? bits0 - 11 : 0; }
 
 template <int LEVEL>
 __global__ __launch_bounds__(kThreads) void member_hist_kernel(
-    const float *__restrict__ p, int64_t n, int64_t k, State *state, const uint32_t *hist_prev,
-    uint32_t *__restrict__ hist_out, uint32_t *boff, uint32_t *wg_bins, int seg_shift,
+    const float *__restrict__ p, int64_t n, int64_t k, int mid_bins, State *state,
+    const uint32_t *hist_prev, uint32_t *__restrict__ hist_out, const uint32_t *histf_prev,
+    uint32_t *__restrict__ histf_out, uint32_t *boff, uint32_t *wg_bins, int seg_shift,
     int64_t wave_len, const uint32_t *__restrict__ wave_listed,
     const uint64_t *__restrict__ lists, int list_cap) {
-  __shared__ uint32_t h[kBinsR];
+  __shared__ uint32_t hp[kBinsF / 2];  // packed counters after a failed hint; else h, below
+  uint32_t *h = hp;
+  static_assert(kBinsR <= kBinsF / 2, "the level's histogram fits the same LDS");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int i = tid; i < kBinsR; i += kThreads) h[i] = 0u;
   // the wave's list does not depend on the pick: its length and first stretch are asked for
@@ -726,27 +1028,69 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
   const uint64_t ent_pre = list[lane];
   uint32_t lo, hi;  // the keys that are counted
   int shift;        // digit = (key - lo) >> shift
-  bool full;
+  bool full, fail;
+  uint32_t a_end = 0u, upper16 = 0u;
   // what earlier launches left in the state is asked for before the histogram is walked, not
   // after it (a round trip to memory each time)
   if (LEVEL == 1) {
     const BinMap map = state->map;
     const uint32_t overflow = state->overflow, hint_bin = state->hint_bin;
-    const Pick r = pick_bin<kBins0>((uint32_t)k, hist_prev, boff, wg_bins, seg_shift);
+    const bool hinted = map.uniform == 0u && hint_bin != kNoLists;
+    // (the 2k-th largest key, where the histogram holds that many: the next call's hint)
+    uint32_t bin2 = 0u;
+    // (a hinted call that does not ask for the bins' places in value order has a compact map)
+    const bool compact = hinted && boff == nullptr;
+    const Pick r = compact ? pick_copies((uint32_t)k, hist_prev, map, 2u * (uint32_t)k, &bin2)
+                           : pick_bin<kBins0>((uint32_t)k, hist_prev, boff, wg_bins, seg_shift,
+                                              hinted ? 2u * (uint32_t)k : 0u, &bin2);
+    fail = hinted && r.found == 0u;
     lo = bin_lo_key(map, r.bin);
     hi = bin_hi_key(map, r.bin);
     shift = level1_shift(bits_of(hi - lo));
-    full = overflow != 0u || r.bin < hint_bin;
+    full = overflow != 0u || fail;
+    a_end = map.a_end;
     if (blockIdx.x == 0 && tid == 0) {
       state->prefix[0] = r.bin;
-      state->k_rem[0] = r.k_rem;
+      state->k_rem[0] = fail ? (uint32_t)k - r.total : r.k_rem;
       state->full = full ? 1u : 0u;
+      state->fail = fail ? 1u : 0u;
       state->lo0 = lo;
       state->hi0 = hi;
+      if (hinted && !fail) {
+        // The next call's hint, from exact counts: the coarse-bin boundary at or below the 2k-th
+        // largest key; with fewer than 2k candidates one coarse bin below this call's.
+        const uint32_t step = 1u << kLowShift;
+        uint32_t next = bin2 >= map.nb0 && bin2 != 0u ? bin_lo_key(map, bin2) & ~(step - 1u)
+                                                      : (map.a_end >= step ? map.a_end - step : 0u);
+        state->next_a_end = next;
+        state->next_b_last = map.b_last;
+        state->next_magic = next_mark(n, k, mid_bins);
+      }
+      if (fail && boff != nullptr) {
+        // Value order: the entries below the hint that end up selected follow the r.total
+        // candidates in the output.  Every coarse bin below the hint got boff = r.total above
+        // (all of them lie "above the k-th"), so those entries go to the segment in whose
+        // stretch place r.total lies; that segment's table entry is widened to the coarse bins
+        // [0, nb0) and to the rest of the output.
+        const uint32_t w = r.total >> seg_shift;
+        atomicMax(&wg_bins[4 * w], map.nb0);
+        atomicMax(&wg_bins[4 * w + 1], (uint32_t)kBins0);
+        atomicMax(&wg_bins[4 * w + 2], ~r.total);
+        atomicMax(&wg_bins[4 * w + 3], (uint32_t)k);
+      }
     }
   } else {
     const uint32_t lo0 = state->lo0, hi0 = state->hi0, full0 = state->full;
-    const Pick r = pick_bin<kBinsR>(state->k_rem[0], hist_prev, nullptr);
+    fail = state->fail != 0u;
+    a_end = state->map.a_end;
+    const uint32_t k_rem0 = state->k_rem[0];
+    Pick r;
+    if (!fail) {
+      r = pick_bin<kBinsR>(k_rem0, hist_prev, nullptr);
+    } else {
+      r = pick_wide(k_rem0, histf_prev);
+      upper16 = r.bin;
+    }
     const int shift1 = level1_shift(bits_of(hi0 - lo0));
     lo = lo0 + (r.bin << shift1);
     hi = lo + ((1u << shift1) - 1u);
@@ -759,6 +1103,23 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
     }
   }
   __syncthreads();
+  if (fail) {
+    // the entries below the hint: exactly the ones level 0 did not take for candidates
+    const float lo_f = lower_bound_float(a_end);
+    if (LEVEL == 1) {
+      wide_hist(p, n, wave_len, gw, hp, histf_out, [&](float q, uint32_t *d) {
+        *d = order_key(q) >> 16;
+        return q < lo_f;
+      });
+    } else {
+      wide_hist(p, n, wave_len, gw, hp, histf_out, [&](float q, uint32_t *d) {
+        const uint32_t key = order_key(q);
+        *d = key & 0xffffu;
+        return q < lo_f && (key >> 16) == upper16;
+      });
+    }
+    return;
+  }
   // a wave whose list overflowed reads its own range again, the others walk their lists
   if (!full && m_raw != kListFull) {
     const int m = m_pre;
@@ -795,8 +1156,8 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
 // Packed counts: greater << 32 | equal.  When the levels before streamed the priorities, this
 // launch does too and lists every wave's entries at or above the threshold on the way.
 __global__ __launch_bounds__(kThreads) void count_kernel(
-    const float *__restrict__ p, int64_t n, State *state, const uint32_t *hist2, int64_t wave_len,
-    uint32_t *__restrict__ wave_listed, uint64_t *__restrict__ lists, int list_cap,
+    const float *__restrict__ p, int64_t n, State *state, const uint32_t *hist2,
+    const uint32_t *histf2, int64_t wave_len, uint32_t *__restrict__ wave_listed, uint64_t *__restrict__ lists, int list_cap,
     uint64_t *__restrict__ wave_ge, uint64_t *__restrict__ block_ge) {
   __shared__ uint64_t red[kWavesPerBlock];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -808,8 +1169,15 @@ __global__ __launch_bounds__(kThreads) void count_kernel(
   const uint64_t ent_pre = list[lane];
   const uint32_t lo0 = state->lo0, hi0 = state->hi0, digit1 = state->prefix[1];
   const bool full = state->full != 0u || m_raw == kListFull;  // this wave reads its range
-  const Pick r = pick_bin<kBinsR>(state->k_rem[1], hist2, nullptr);
-  const uint32_t thr = lo0 + (digit1 << level1_shift(bits_of(hi0 - lo0))) + r.bin;
+  const bool fail = state->fail != 0u;  // digit1: the upper 16 bits, histf2: the lower ones
+  const uint32_t k_rem1 = state->k_rem[1];
+  Pick r;
+  if (!fail)
+    r = pick_bin<kBinsR>(k_rem1, hist2, nullptr);
+  else
+    r = pick_wide(k_rem1, histf2);
+  const uint32_t thr = fail ? ((digit1 << 16) | r.bin)
+                            : lo0 + (digit1 << level1_shift(bits_of(hi0 - lo0))) + r.bin;
   if (blockIdx.x == 0 && tid == 0) {
     state->prefix[2] = thr;
     state->k_rem[2] = r.k_rem;
@@ -1580,9 +1948,11 @@ using namespace gearhip;
 
 extern "C" size_t gear_hip_topk_workspace_bytes(int64_t n, int64_t k) { return layout(n, k).total; }
 
-extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
-                                 int sorted_by_value, float *values_out, int64_t *indices_out,
-                                 void *workspace, size_t workspace_bytes, void *stream) {
+namespace gearhip {
+namespace {
+int topk_launch(const float *priorities, int64_t n, int64_t k, int sorted_by_value, int warm,
+                float *values_out, int64_t *indices_out, void *workspace, size_t workspace_bytes,
+                void *stream) {
   if (n < 0 || k < 0) return GEAR_HIP_EINVAL;
   if (k == 0) return 0;
   if (k > n || !priorities || !indices_out) return GEAR_HIP_EINVAL;
@@ -1596,6 +1966,8 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   uint32_t *hist0 = reinterpret_cast<uint32_t *>(ws + l.hist0);
   uint32_t *hist1 = reinterpret_cast<uint32_t *>(ws + l.hist1);
   uint32_t *hist2 = reinterpret_cast<uint32_t *>(ws + l.hist2);
+  uint32_t *histf1 = reinterpret_cast<uint32_t *>(ws + l.histf1);
+  uint32_t *histf2 = reinterpret_cast<uint32_t *>(ws + l.histf2);
   uint32_t *boff = reinterpret_cast<uint32_t *>(ws + l.boff);
   uint32_t *wave_listed = reinterpret_cast<uint32_t *>(ws + l.wave_listed);
   uint64_t *wave_ge = reinterpret_cast<uint64_t *>(ws + l.wave_ge);
@@ -1645,31 +2017,39 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
     uint32_t *zero = reinterpret_cast<uint32_t *>(ws + l.zero_begin);
     const dim3 pgrid(1 + zero_blocks);
     if (per == 2)
-      prep_kernel<2><<<pgrid, block, 0, st>>>(priorities, n, rank, list_all, mid_bins, state, zero,
-                                              zero_words);
+      prep_kernel<2><<<pgrid, block, 0, st>>>(priorities, n, k, rank, list_all, mid_bins, warm, state,
+                                              zero, zero_words);
     else if (per == 8)
-      prep_kernel<8><<<pgrid, block, 0, st>>>(priorities, n, rank, list_all, mid_bins, state, zero,
-                                              zero_words);
+      prep_kernel<8><<<pgrid, block, 0, st>>>(priorities, n, k, rank, list_all, mid_bins, warm, state,
+                                              zero, zero_words);
     else
-      prep_kernel<32><<<pgrid, block, 0, st>>>(priorities, n, rank, list_all, mid_bins, state,
+      prep_kernel<32><<<pgrid, block, 0, st>>>(priorities, n, k, rank, list_all, mid_bins, warm, state,
                                                zero, zero_words);
   }
-  level0_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len, wave_listed,
-                                        lists, (int)g.list_cap);
+  if (rank != 0u && mid_bins == kMidBinsCoarse)
+    level0_hinted_kernel<true><<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len,
+                                                       wave_listed, lists, (int)g.list_cap);
+  else if (rank != 0u)
+    level0_hinted_kernel<false><<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len,
+                                                        wave_listed, lists, (int)g.list_cap);
+  else
+    level0_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len, wave_listed,
+                                          lists, (int)g.list_cap);
   // value order by segments: workgroup w of the sort owns the bins that start in the output
   // places [w << seg_shift, (w + 1) << seg_shift)
   const bool by_segments = sorted_by_value && k <= kBucketMaxK;
   int seg_shift = 0;
   while ((k >> seg_shift) >= kNoSegment) ++seg_shift;  // segment ids stay below kNoSegment
   uint32_t *wg_bins = reinterpret_cast<uint32_t *>(ws + l.wg_bins);
-  member_hist_kernel<1><<<grid, block, 0, st>>>(priorities, n, k, state, hist0, hist1,
-                                                by_segments ? boff : nullptr, wg_bins, seg_shift,
-                                                g.wave_len, wave_listed, lists, (int)g.list_cap);
-  member_hist_kernel<2><<<grid, block, 0, st>>>(priorities, n, k, state, hist1, hist2, nullptr,
-                                                nullptr, 0, g.wave_len, wave_listed, lists,
+  member_hist_kernel<1><<<grid, block, 0, st>>>(priorities, n, k, mid_bins, state, hist0, hist1,
+                                                nullptr, histf1, by_segments ? boff : nullptr,
+                                                wg_bins, seg_shift, g.wave_len, wave_listed, lists,
                                                 (int)g.list_cap);
-  count_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist2, g.wave_len, wave_listed, lists,
-                                       (int)g.list_cap, wave_ge, block_ge);
+  member_hist_kernel<2><<<grid, block, 0, st>>>(priorities, n, k, mid_bins, state, hist1, hist2,
+                                                histf1, histf2, nullptr, nullptr, 0, g.wave_len,
+                                                wave_listed, lists, (int)g.list_cap);
+  count_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist2, histf2, g.wave_len,
+                                       wave_listed, lists, (int)g.list_cap, wave_ge, block_ge);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   uint8_t *cseg = reinterpret_cast<uint8_t *>(ws + l.cseg);
 #define GEARHIP_WRITE(F, CKEY)                                                                     \
@@ -1704,4 +2084,21 @@ extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
   const EmitSorted fin{priorities, values_out, indices_out, (uint32_t)n};
   return radix::sort_pairs<uint32_t, uint32_t, EmitSorted>(ckey, skey, cidx, sidx, tkey, tidx, k, 0,
                                                            32, shist, st, fin);
+}
+}  // namespace
+}  // namespace gearhip
+
+extern "C" int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k,
+                                 int sorted_by_value, float *values_out, int64_t *indices_out,
+                                 void *workspace, size_t workspace_bytes, void *stream) {
+  return topk_launch(priorities, n, k, sorted_by_value, 0, values_out, indices_out, workspace,
+                     workspace_bytes, stream);
+}
+
+extern "C" int gear_hip_topk_f32_warm(const float *priorities, int64_t n, int64_t k,
+                                      int sorted_by_value, float *values_out,
+                                      int64_t *indices_out, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+  return topk_launch(priorities, n, k, sorted_by_value, 1, values_out, indices_out, workspace,
+                     workspace_bytes, stream);
 }

@@ -371,16 +371,44 @@ def sort_i64(keys, vals=None, key_bits=63):
     return (keys_out, vals_out) if vals is not None else keys_out
 
 
-def topk(priorities, k, *, sorted_by_value=True, want_values=True):
+def topk(priorities, k, *, sorted_by_value=True, want_values=True, warm=False, workspace=None):
+    """Top-k of fp32 priorities (values, indices), by value descending or by index ascending.
+    warm=True: the call may start from the bound that the last call on `workspace` (same n, k and
+    order) left there instead of sampling the array; the result is the same either way."""
     _need(priorities, torch.float32, "priorities")
     n = priorities.numel()
     idx = torch.empty(k, dtype=torch.int64, device=priorities.device)
     vals = torch.empty(k, dtype=torch.float32, device=priorities.device) if want_values else None
     nbytes = load().gear_hip_topk_workspace_bytes(n, k)
-    ws = _ws.get("topk", nbytes, priorities.device)
-    call("gear_hip_topk_f32", _ptr(priorities), n, int(k), int(bool(sorted_by_value)), _ptr(vals),
-         _ptr(idx), _ptr(ws), ws.numel(), _stream())
+    ws = workspace if workspace is not None else _ws.get("topk", nbytes, priorities.device)
+    if ws.numel() < nbytes:
+        raise ValueError("top-k workspace holds %d bytes, %d needed" % (ws.numel(), nbytes))
+    call("gear_hip_topk_f32_warm" if warm else "gear_hip_topk_f32", _ptr(priorities), n, int(k),
+         int(bool(sorted_by_value)), _ptr(vals), _ptr(idx), _ptr(ws), ws.numel(), _stream())
     return vals, idx
+
+
+class TopKState:
+    """A top-k selection that is repeated on one slowly changing priority array (the priority
+    maintenance of a replay buffer): owns the workspace, so that every call after the first can
+    take up the bound the call before it left (gear_hip_topk_f32_warm)."""
+
+    def __init__(self):
+        self._ws = None
+        self._shape = None
+
+    def select(self, priorities, k, *, sorted_by_value=True, want_values=True):
+        n = priorities.numel()
+        shape = (n, int(k), bool(sorted_by_value), priorities.device)
+        nbytes = load().gear_hip_topk_workspace_bytes(n, k)
+        warm = self._shape == shape
+        if self._ws is None or self._ws.numel() < nbytes or self._ws.device != priorities.device:
+            self._ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8,
+                                   device=priorities.device)
+            warm = False
+        self._shape = shape
+        return topk(priorities, k, sorted_by_value=sorted_by_value, want_values=want_values,
+                    warm=warm, workspace=self._ws)
 
 
 def scatter(weights, idx, values, *, unique_indices=False):

@@ -316,14 +316,30 @@ int gear_hip_sort_i64(const int64_t *keys_in, int64_t *keys_out, const int64_t *
  * The priorities are normally read once: a sample of 2048 of them places a bound safely below
  * the k-th largest, the one pass over the array lists everything above the bound, and the exact
  * selection runs on those lists.  Where a list overflows (clustered maxima, masses of ties) the
- * later steps read that part of the array again, where the bound fails all of it; the result is
- * the same either way.
+ * later steps read that part of the array again; where the bound fails (fewer than k entries
+ * above it: a sample that misleads) two of them read all of it again and look for the threshold
+ * among the entries below the bound.  The result is the same either way.
  * workspace: gear_hip_topk_workspace_bytes(n, k) bytes on the device, 256-byte aligned; its
  * contents need not be initialised (the call clears what it needs on `stream`). */
 size_t gear_hip_topk_workspace_bytes(int64_t n, int64_t k);
 int gear_hip_topk_f32(const float *priorities, int64_t n, int64_t k, int sorted_by_value,
                       float *values_out, int64_t *indices_out, void *workspace,
                       size_t workspace_bytes, void *stream);
+
+/* The same selection for a caller that repeats it on a slowly changing array (the priority
+ * maintenance of a replay buffer between batches: TopKSampler.sync_sample on every step,
+ * gear/sampler/global_sampler.py:175-203, after the updates of src/index/request.cc:41-51).
+ * Every call leaves in the workspace the bound the NEXT call can start from: the boundary at or
+ * below the 2k-th largest priority, taken from this call's exact counts.  This form takes that
+ * bound up instead of drawing a sample when `workspace` was last used by gear_hip_topk_f32 or
+ * this function with the same n, k and order (a mark in the workspace says so; anything else in
+ * it, and a call whose own bound failed, lead to a sample as in gear_hip_topk_f32).  The bound
+ * only decides how the work is done: however stale it is, the result equals gear_hip_topk_f32's
+ * bit for bit (too high: the entries below it are searched as described above; too low: lists
+ * overflow and those parts of the array are read again). */
+int gear_hip_topk_f32_warm(const float *priorities, int64_t n, int64_t k, int sorted_by_value,
+                           float *values_out, int64_t *indices_out, void *workspace,
+                           size_t workspace_bytes, void *stream);
 
 /* Priority update  weights[idx[j]] = values[j], j in [0,num).
  * Replaces the host loop over Indexset::set_weight (include/index/set.h:245-247) and fixes the

@@ -260,6 +260,76 @@ def test_topk_with_a_misleading_sample(oracle):
     _check_topk(oracle, ops, neg, 30_000, "all negative")
 
 
+def _check_state(oracle, state, w, k, by_value, label):
+    announce("warm topk %s n=%d k=%d by_value=%d" % (label, len(w), k, by_value))
+    vals, idx = state.select(_dev(w), k, sorted_by_value=by_value)
+    torch.cuda.synchronize()
+    evals, eidx = oracle.topk_f32(w, k, by_value)
+    assert np.array_equal(idx.cpu().numpy(), eidx), label
+    assert np.array_equal(vals.cpu().numpy().view(np.uint32), w[eidx].view(np.uint32)), label
+
+
+@pytest.mark.parametrize("by_value", [True, False])
+def test_topk_warm_calls_follow_a_changing_array(oracle, by_value):
+    """The warm form starts from the bound the call before it left in the workspace.  The bound
+    only decides how the work is done: on an array that changes a little between calls (the
+    replay buffer's priority updates), on one whose priorities all shrank (the stale bound is
+    too high: fewer than k entries above it), on one whose priorities all grew (too low: the
+    lists overflow), and after a call of another shape, the result is the oracle's."""
+    from gear_amd import ops
+    rng = np.random.default_rng(91)
+    n, k = 2_000_000, 65_536
+    w = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    state = ops.TopKState()
+    _check_state(oracle, state, w, k, by_value, "first call (a sample)")
+    for step in range(3):
+        pos = rng.permutation(n)[:20_000]
+        w[pos] = (rng.lognormal(0, 1, size=pos.size) ** 0.6).astype(np.float32)
+        _check_state(oracle, state, w, k, by_value, "after updates %d" % step)
+    small = (w * np.float32(0.01)).astype(np.float32)
+    _check_state(oracle, state, small, k, by_value, "all priorities shrank (bound too high)")
+    _check_state(oracle, state, small, k, by_value, "the call after the failed bound")
+    _check_state(oracle, state, small, k, by_value, "and the one after that")
+    big = (w * np.float32(100.0)).astype(np.float32)
+    _check_state(oracle, state, big, k, by_value, "all priorities grew (bound too low)")
+    _check_state(oracle, state, big, k, by_value, "the call after the overflow")
+    _check_state(oracle, state, big, k, by_value, "and the one after that")
+    _check_state(oracle, state, w[:1_500_000].copy(), 30_000, by_value, "another shape")
+    _check_state(oracle, state, w[:1_500_000].copy(), 30_000, by_value, "the same shape again")
+    # a bound just above most of the array: few candidates, the k-th largest far below it
+    spike = w.copy()
+    spike[rng.permutation(n)[:200_000]] += np.float32(50.0)
+    _check_state(oracle, state, spike, 150_000 if not by_value else 100_000, by_value,
+                 "a fifth of a million entries lifted")
+    plain = w.copy()
+    _check_state(oracle, state, plain, 150_000 if not by_value else 100_000, by_value,
+                 "and dropped again (bound too high by far)")
+
+
+def test_topk_warm_on_a_workspace_that_holds_something_else(oracle):
+    """A warm call on a workspace that no top-k call has used (zeros, ones, the prefix sums of an
+    earlier tenant) finds no mark and draws its sample like the plain form."""
+    from gear_amd import ops, _cabi
+    lib = _cabi.load()
+    rng = np.random.default_rng(92)
+    n, k = 1_000_000, 10_000
+    w = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    nbytes = lib.gear_hip_topk_workspace_bytes(n, k)
+    evals, eidx = oracle.topk_f32(w, k, True)
+    for fill in ("zeros", "ones", "ramp"):
+        announce("warm topk on a workspace of %s" % fill)
+        if fill == "zeros":
+            ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        elif fill == "ones":
+            ws = torch.full((nbytes,), 255, dtype=torch.uint8, device="cuda")
+        else:
+            ws = torch.arange(nbytes // 8 + 1, dtype=torch.int64, device="cuda").view(torch.uint8)[:nbytes].clone()
+        vals, idx = ops.topk(_dev(w), k, sorted_by_value=True, warm=True, workspace=ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(idx.cpu().numpy(), eidx)
+        assert np.array_equal(vals.cpu().numpy().view(np.uint32), evals.view(np.uint32))
+
+
 def test_topk_config5_size(oracle):
     """Config 5's maintenance step at full size: top-65 536 of 10 000 000 lognormal^0.6."""
     from gear_amd import ops
