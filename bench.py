@@ -243,7 +243,100 @@ def run_config4(args):
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst)
+    if not args.no_hostlink:
+        # after everything the line is made of has been measured: the same batch shape gathered
+        # from a pinned host table (config 5's zero-copy path) against the host link
+        del table
+        torch.cuda.empty_cache()
+        try:
+            result["config5_hostlink"] = config5_hostlink(np, torch, ops, args.hostlink_trajectories)
+        except Exception as exc:  # a refused pin or anything else here never fails the bench
+            log("config-5 host-link sub-record skipped: %r" % (exc,))
+            result["config5_hostlink"] = None
     return result
+
+
+def config5_hostlink(np, torch, ops, cap):
+    """Bounded sub-record of the config-4 line: config 5's gather -- 2048 windows x 30 steps x 4
+    columns read by the GPU in place from a pinned, mapped host table -- next to a pinned
+    hipMemcpyAsync host-to-device copy of the same number of bytes in the same run (the method of
+    the reference's own benchmark, examples/offline/single-node/misc.py:34-46, on the path of
+    src/storage/handler.cc:148-153).  The table is smaller than config 5's 56 GB: what the link
+    delivers does not depend on the size of the table the windows are spread over."""
+    import ctypes
+    from gear_amd import _cabi
+    lib = _cabi.load()
+    T, B, span, ofst = 1000, 2048, 30, -29
+    tab = AtariTable(T, cap)
+    host_ptr, dev_ptr = ctypes.c_void_p(), ctypes.c_void_p()
+    log("pinning %.1f GB of host memory for the host-link sub-record" % (tab.nbytes / 1e9))
+    rc = lib.gear_hip_host_alloc(tab.nbytes, ctypes.byref(host_ptr), ctypes.byref(dev_ptr))
+    if rc != 0:
+        raise RuntimeError("gear_hip_host_alloc(%d) returned %d" % (tab.nbytes, rc))
+    try:
+        g = torch.Generator(device="cuda")
+        g.manual_seed(1005)
+        piece = torch.randint(0, 256, (1 << 28,), dtype=torch.uint8, device="cuda", generator=g)
+        for o in range(0, tab.nbytes, piece.numel()):
+            nb = min(piece.numel(), tab.nbytes - o)
+            _cabi.call("gear_hip_memcpy", ctypes.c_void_p(host_ptr.value + o),
+                       ctypes.c_void_p(piece.data_ptr()), nb)
+        del piece
+        flat = torch.sort(torch.randint(0, T * cap, (B,), dtype=torch.int64, device="cuda",
+                                        generator=g)).values
+        idxs, tss = flat // T, flat % T
+        lens = tss + 1
+        dsts = [torch.empty((B, span * sb), dtype=torch.uint8, device="cuda")
+                for sb in tab.step_bytes]
+        cols = [dict(dst=dsts[c], ofst=ofst, span=span, step_bytes=tab.step_bytes[c],
+                     col_base=tab.col_base(c), pad_head=True, zero_fill=True) for c in range(4)]
+        payload = B * span * sum(tab.step_bytes)
+        read_bytes = int(torch.clamp(tss + 1, max=span).sum().item()) * sum(tab.step_bytes)
+
+        def timed_ms(fn, warm, reps):
+            for _ in range(warm):
+                fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / reps
+
+        gather_ms = timed_ms(lambda: ops.subcopy_multi(dev_ptr.value, idxs, tss, lens,
+                                                       tab.traj_stride, cols), 3, 10)
+        # a window is checked against the host bytes it came from
+        w = B // 2
+        i, ts = int(idxs[w].item()), int(tss[w].item())
+        n = min(ts + 1, span)
+        for c in (0, 3):
+            sb = tab.step_bytes[c]
+            off = i * tab.traj_stride + tab.col_base(c) + (ts + 1 - n) * sb
+            src = np.ctypeslib.as_array(ctypes.cast(host_ptr.value + off,
+                                                    ctypes.POINTER(ctypes.c_uint8)), shape=(n * sb,))
+            got = dsts[c][w].cpu().numpy()
+            if not (np.array_equal(got[(span - n) * sb:], src) and not got[:(span - n) * sb].any()):
+                raise RuntimeError("host-table gather does not match the host bytes")
+        pin = torch.empty(read_bytes, dtype=torch.uint8, pin_memory=True)
+        dev = torch.empty(read_bytes, dtype=torch.uint8, device="cuda")
+        h2d_ms = timed_ms(lambda: dev.copy_(pin, non_blocking=True), 2, 5)
+        achieved = read_bytes / (gather_ms * 1e-3) / 1e9
+        peak = read_bytes / (h2d_ms * 1e-3) / 1e9
+        return {"bound": "host-link", "kernel": "subcopy_multi_kernel (source in pinned host memory)",
+                "achieved": achieved, "peak": peak, "unit": "GB/s", "frac": achieved / peak,
+                "peak_source": "pinned hipMemcpyAsync host-to-device copy of the same bytes, same run",
+                "table_bytes": tab.nbytes, "bytes_over_the_link_per_launch": read_bytes,
+                "batch_payload_bytes": payload,
+                "parts_ms": {"gather": gather_ms, "h2d_copy": h2d_ms},
+                "windows_per_s": B / (gather_ms * 1e-3),
+                "what": "10 zero-copy gathers of 2048 windows x 30 steps x 4 columns from a %d-"
+                        "trajectory (%.2f GB) Atari-shape table in pinned host memory; 5 pinned "
+                        "host-to-device copies of the bytes those windows read"
+                        % (cap, tab.nbytes / 1e9)}
+    finally:
+        lib.gear_hip_host_free(host_ptr)
 
 
 def cpu_baseline_config4(np, torch, tab, table, pri, B, span, ofst):
@@ -679,6 +772,7 @@ def run_config5(args):
     cols = [dict(dst=dsts[c], ofst=ofst, span=span, step_bytes=tab.step_bytes[c],
                  col_base=tab.col_base(c), pad_head=True) for c in range(4)]
     names = ["scatter", "topk", "scan", "sample", "gather"]
+    selection = ops.TopKState()   # steps after the first start from the last step's bound
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)]
           for _ in range(args.steps)]
 
@@ -687,7 +781,7 @@ def run_config5(args):
         if e: e[0].record()
         ops.scatter(pri, upd_idx[i % 4], upd_val[i % 4], unique_indices=True)
         if e: e[1].record()
-        ops.topk(pri, k, sorted_by_value=True)
+        selection.select(pri, k, sorted_by_value=True)
         if e: e[2].record()
         ops.prefix_sum(pri, out=prefix)
         if e: e[3].record()
@@ -891,10 +985,19 @@ def run_topk(args):
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(args.steps)]
 
+    # --topk-warm: every call after the first starts from the bound the call before it left in the
+    # workspace (gear_hip_topk_f32_warm), as a loop over a slowly changing array does
+    state = ops.TopKState() if args.topk_warm else None
+
+    def select():
+        if state is not None:
+            return state.select(pri, k, sorted_by_value=by_value)
+        return ops.topk(pri, k, sorted_by_value=by_value)
+
     def step(i, slot):
         if slot is not None:
             ev[slot][0].record()
-        ops.topk(pri, k, sorted_by_value=by_value)
+        select()
         if slot is not None:
             ev[slot][1].record()
 
@@ -914,13 +1017,14 @@ def run_topk(args):
         torch.cuda.synchronize()
         return a.elapsed_time(b) / reps * 1e3
 
-    yard = {"back_to_back_us": timed_us(lambda: ops.topk(pri, k, sorted_by_value=by_value)),
+    yard = {"back_to_back_us": timed_us(select),
             "torch_topk_us": timed_us(lambda: torch.topk(pri, k, sorted=by_value), reps=10),
             "torch_sum_read_only_us": timed_us(lambda: pri.sum()),
             "what": "HIP events around back-to-back launches, same n and k; torch.topk is the "
-                    "library selection, pri.sum() one read of the priorities"}
+                    "library selection, pri.sum() one read of the priorities (two launches)"}
     return _line(n / (ms * 1e-3), "priorities/s", args, ms,
-                 "topk: top %d of %d fp32 priorities, ordered by %s" % (k, n, args.topk_order),
+                 "topk: top %d of %d fp32 priorities, ordered by %s%s" %
+                 (k, n, args.topk_order, ", warm calls" if args.topk_warm else ""),
                  {"bound": "hbm", "kernel": "top-k chain (prep, level0, member_hist x2, count, "
                                             "write" + (", segment_sort)" if by_value else ")"),
                   "achieved": alg / (avg * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -942,7 +1046,13 @@ def main():
                          "one maintenance kernel chain on its own, for profiles")
     ap.add_argument("--n", type=int, default=10_000_000, help="scan / topk: number of priorities")
     ap.add_argument("--k", type=int, default=65_536, help="topk: entries kept")
+    ap.add_argument("--no-hostlink", action="store_true",
+                    help="config4: skip the bounded config-5 host-link sub-record")
+    ap.add_argument("--hostlink-trajectories", type=int, default=150,
+                    help="config4: trajectories (28.2 MB each) of the pinned table of that sub-record")
     ap.add_argument("--topk-order", default="value", choices=["value", "index"])
+    ap.add_argument("--topk-warm", action="store_true",
+                    help="topk: calls after the first take up the previous call's bound")
     ap.add_argument("--trajectories3", type=int, default=100_000,
                     help="config 3: number of trajectories (100000 = full size, 10.4 GB)")
     ap.add_argument("--trajectories5", type=int, default=2000,

@@ -73,6 +73,14 @@ SIGNATURES = {
     "gear_hip_sample_sorted_f64": (c_int, [c_void_p, c_i64, c_void_p, c_i64, c_int, c_void_p, c_i64,
                                            c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                            c_void_p]),
+    "gear_hip_sample_lookup_f64": (c_int, [c_void_p, c_i64, c_void_p, c_i64, c_int, c_void_p, c_i64,
+                                           c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_size_t, c_void_p]),
+    "gear_hip_sort_lookup_i64": (c_int, [c_void_p, c_i64, c_i64, c_void_p, c_i64, c_i64, c_void_p,
+                                         c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                         c_void_p]),
+    "gear_hip_lookup_i64": (c_int, [c_void_p, c_i64, c_void_p, c_i64, c_i64, c_void_p, c_i64,
+                                    c_void_p, c_void_p, c_void_p, c_void_p]),
     "gear_hip_upper_bound_i64": (c_int, [c_void_p, c_i64, c_void_p, c_i64, c_int, c_void_p,
                                          c_void_p]),
     "gear_hip_sort_workspace_bytes": (c_size_t, [c_i64]),

@@ -238,6 +238,40 @@ struct Handler {
       : table(t), impl(t, g, w, r) {}
 };
 
+// the column descriptors of one multi-column gather of `num` windows into dsts (and masks)
+std::vector<gear_hip_column_desc> column_descs(Handler &h, int64_t num,
+                                               const std::vector<size_t> &columns,
+                                               const std::vector<py::object> &dsts, bool zero_fill,
+                                               const py::object &masks) {
+  if (columns.size() != dsts.size() || columns.size() > GEAR_HIP_MAX_COLUMNS)
+    throw std::runtime_error("columns and dsts differ in length (or more than 16 columns)");
+  std::vector<gear_hip_column_desc> descs(columns.size());
+  for (size_t k = 0; k < columns.size(); ++k) {
+    const ColumnWindow w = h.impl.window(columns[k]);
+    TensorInfo d = tensor_info(dsts[k], "dst", 0, 1);
+    if (d.numel * d.elem < num * w.dst_stride)
+      throw std::runtime_error("dst is smaller than the gathered batch");
+    descs[k].dst = d.ptr;
+    descs[k].mask_out = nullptr;
+    if (!masks.is_none()) {
+      py::object mk = masks.cast<py::sequence>()[k];
+      if (!mk.is_none()) {
+        TensorInfo mi = tensor_info(mk, "mask", 1, 1);
+        if (mi.numel < num * w.span) throw std::runtime_error("mask is smaller than [num, length]");
+        descs[k].mask_out = static_cast<uint8_t *>(mi.ptr);
+      }
+    }
+    descs[k].ofst = w.ofst;
+    descs[k].span = w.span;
+    descs[k].step_bytes = w.step_bytes;
+    descs[k].col_base = w.col_base;
+    descs[k].dst_stride = w.dst_stride;
+    descs[k].pad_head = w.pad_head ? 1 : 0;
+    descs[k].zero_fill = zero_fill ? 1 : 0;
+  }
+  return descs;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_libgear, libgear) {
@@ -499,32 +533,8 @@ PYBIND11_MODULE(_libgear, libgear) {
                         c = tensor_info(lens, "lengths", 8, 1);
              if (a.numel != b.numel || a.numel != c.numel)
                throw std::runtime_error("indices, timesteps and lengths differ in size");
-             if (columns.size() != dsts.size() || columns.size() > GEAR_HIP_MAX_COLUMNS)
-               throw std::runtime_error("columns and dsts differ in length (or more than 16 columns)");
-             std::vector<gear_hip_column_desc> descs(columns.size());
-             for (size_t k = 0; k < columns.size(); ++k) {
-               const ColumnWindow w = h.impl.window(columns[k]);
-               TensorInfo d = tensor_info(dsts[k], "dst", 0, 1);
-               if (d.numel * d.elem < a.numel * w.dst_stride)
-                 throw std::runtime_error("dst is smaller than the gathered batch");
-               descs[k].dst = d.ptr;
-               descs[k].mask_out = nullptr;
-               if (!masks.is_none()) {
-                 py::object mk = masks.cast<py::sequence>()[k];
-                 if (!mk.is_none()) {
-                   TensorInfo mi = tensor_info(mk, "mask", 1, 1);
-                   if (mi.numel < a.numel * w.span) throw std::runtime_error("mask is smaller than [num, length]");
-                   descs[k].mask_out = static_cast<uint8_t *>(mi.ptr);
-                 }
-               }
-               descs[k].ofst = w.ofst;
-               descs[k].span = w.span;
-               descs[k].step_bytes = w.step_bytes;
-               descs[k].col_base = w.col_base;
-               descs[k].dst_stride = w.dst_stride;
-               descs[k].pad_head = w.pad_head ? 1 : 0;
-               descs[k].zero_fill = zero_fill ? 1 : 0;
-             }
+             const std::vector<gear_hip_column_desc> descs =
+                 column_descs(h, a.numel, columns, dsts, zero_fill, masks);
              check_hip("subcopy_multi",
                        gear_hip_subcopy_multi_checked(
                            h.impl.device_base(), a.numel, static_cast<const int64_t *>(a.ptr),
@@ -536,6 +546,84 @@ PYBIND11_MODULE(_libgear, libgear) {
            },
            py::arg("indices"), py::arg("timesteps"), py::arg("lengths"), py::arg("columns"),
            py::arg("dsts"), py::arg("zero_fill") = true, py::arg("masks") = py::none())
+      // One call for a loader step after the draws (no reference counterpart as a binding: it is
+      // OfflineLoader.fused_iterate, gear/loader/offline_loader.py:155-204, from the sort of the
+      // sampled indices to the last column's subcopy): the batch is selected and looked up --
+      //   kind "weighted"   draws = fp32 uniforms in [0, 1), searched in `prefix` (fp64)
+      //   kind "uniform"    draws = int64 positions into `indices`
+      //   kind "positions"  draws = int64 positions already in batch order (a top-k selection)
+      // sorted (not for "positions"), sampled = indices[position], local = sampled - index_offset,
+      // lens = timesteps[local] -- and all columns are gathered with the offline convention
+      // timestep == length (offline_loader.py:200-201), everything enqueued on the current stream.
+      // `indices` must ascend (then sorting positions sorts the sampled indices).
+      .def("select_subcopy",
+           [](Handler &h, const std::string &kind, const py::object &draws, const py::object &prefix,
+              const py::object &indices, int64_t index_offset, const py::object &timesteps,
+              const std::vector<size_t> &columns, const std::vector<py::object> &dsts, bool zero_fill,
+              const py::object &masks, const py::object &sampled_out, const py::object &local_out,
+              const py::object &lens_out) {
+             TensorInfo it = tensor_info(indices, "indices", 8, 1),
+                        tt = tensor_info(timesteps, "timesteps", 8, 1),
+                        so = tensor_info(sampled_out, "sampled_out", 8, 1),
+                        lo = tensor_info(local_out, "local_out", 8, 1),
+                        le = tensor_info(lens_out, "lens_out", 8, 1);
+             void *st = current_stream();
+             int64_t num = 0;
+             if (kind == "weighted") {
+               TensorInfo d = tensor_info(draws, "draws", 4, 1), p = tensor_info(prefix, "prefix", 8, 1);
+               num = d.numel;
+               if (p.numel != it.numel) throw std::runtime_error("prefix and indices differ in length");
+               if (so.numel < num || lo.numel < num || le.numel < num)
+                 throw std::runtime_error("an output is smaller than the batch");
+               size_t have = 0;
+               void *ws = workspace("sample", st, gear_hip_sample_workspace_bytes(num), &have);
+               check_hip("select_subcopy (sample)",
+                         gear_hip_sample_lookup_f64(
+                             static_cast<const double *>(p.ptr), p.numel, static_cast<const float *>(d.ptr),
+                             num, 1, static_cast<const int64_t *>(it.ptr), index_offset,
+                             static_cast<const int64_t *>(tt.ptr), tt.numel, static_cast<int64_t *>(so.ptr),
+                             static_cast<int64_t *>(lo.ptr), static_cast<int64_t *>(le.ptr), ws, have, st));
+             } else if (kind == "uniform" || kind == "positions") {
+               TensorInfo d = tensor_info(draws, "draws", 8, 1);
+               num = d.numel;
+               if (so.numel < num || lo.numel < num || le.numel < num)
+                 throw std::runtime_error("an output is smaller than the batch");
+               if (kind == "uniform") {
+                 size_t have = 0;
+                 void *ws = workspace("sample", st, gear_hip_sample_workspace_bytes(num), &have);
+                 check_hip("select_subcopy (sort)",
+                           gear_hip_sort_lookup_i64(
+                               static_cast<const int64_t *>(d.ptr), num, it.numel > 0 ? it.numel : 1,
+                               static_cast<const int64_t *>(it.ptr), it.numel, index_offset,
+                               static_cast<const int64_t *>(tt.ptr), tt.numel, static_cast<int64_t *>(so.ptr),
+                               static_cast<int64_t *>(lo.ptr), static_cast<int64_t *>(le.ptr), ws, have, st));
+               } else {
+                 check_hip("select_subcopy (look-up)",
+                           gear_hip_lookup_i64(static_cast<const int64_t *>(d.ptr), num,
+                                               static_cast<const int64_t *>(it.ptr), it.numel, index_offset,
+                                               static_cast<const int64_t *>(tt.ptr), tt.numel,
+                                               static_cast<int64_t *>(so.ptr), static_cast<int64_t *>(lo.ptr),
+                                               static_cast<int64_t *>(le.ptr), st));
+               }
+             } else {
+               throw std::invalid_argument("kind must be 'weighted', 'uniform' or 'positions'");
+             }
+             if (num == 0) return;
+             const std::vector<gear_hip_column_desc> descs =
+                 column_descs(h, num, columns, dsts, zero_fill, masks);
+             check_hip("select_subcopy (gather)",
+                       gear_hip_subcopy_multi_checked(
+                           h.impl.device_base(), num, static_cast<const int64_t *>(lo.ptr),
+                           static_cast<const int64_t *>(le.ptr), static_cast<const int64_t *>(le.ptr),
+                           (int64_t)h.impl.table().trajectory_stride(),
+                           (int64_t)h.impl.table().table_spec().capacity,
+                           (int64_t)h.impl.table().table_spec().trajectory_length, descs.data(),
+                           (int)descs.size(), st));
+           },
+           py::arg("kind"), py::arg("draws"), py::arg("prefix"), py::arg("indices"),
+           py::arg("index_offset"), py::arg("timesteps"), py::arg("columns"), py::arg("dsts"),
+           py::arg("zero_fill"), py::arg("masks"), py::arg("sampled_out"), py::arg("local_out"),
+           py::arg("lens_out"))
       .def("view",
            [](Handler &h, size_t index, size_t column) {
              size_t off, len;

@@ -155,6 +155,48 @@ __global__ __launch_bounds__(kBlock) void split_sorted_kernel(const int64_t *__r
   if (lens) lens[j] = ts + 1;
 }
 
+// What the loader does with a sorted batch of positions before it can gather
+// (gear/loader/offline_loader.py:168-177 and the samplers' concat_indices[draws],
+// gear/sampler/global_sampler.py:131,172,196), for the entry at sorted place r with position p:
+//     sampled[r] = index_table ? index_table[p] : p        the batch's global trajectory index
+//     local[r]   = sampled[r] - index_offset               its index in this shard's table
+//     lens[r]    = lengths_table[local[r]]                  its recorded length (0 outside the table)
+struct Lookup {
+  const int64_t *index_table;
+  int64_t index_n, index_offset;
+  const int64_t *lengths_table;
+  int64_t lengths_n;
+  int64_t *sampled, *local, *lens;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t p) const {
+    int64_t g = p;
+    if (index_table) g = (p >= 0 && p < index_n) ? index_table[p] : 0;
+    const int64_t l = g - index_offset;
+    if (sampled) sampled[r] = g;
+    if (local) local[r] = l;
+    if (lens) lens[r] = (lengths_table && l >= 0 && l < lengths_n) ? lengths_table[l] : 0;
+  }
+};
+
+// The ranking sort over a batch of positions (at most kRankMax, each below 2^32), with the
+// look-ups of the sorted entry done by the thread that ranked it: one launch instead of a sort
+// and two gathers.
+__global__ __launch_bounds__(radix::kRankBlock) void rank_lookup_kernel(
+    const int64_t *__restrict__ raw, int num, Lookup look) {
+  typedef uint32_t K;
+  __shared__ radix::RankSmem<K> sm;
+  K mine;
+  const uint32_t rank = radix::block_rank<K>(sm, num, [&](int j) { return (K)raw[j]; }, &mine);
+  const int e = (int)blockIdx.x * kWave + (threadIdx.x & 63);
+  if (threadIdx.x >= kWave || e >= num) return;
+  look((int64_t)rank, (int64_t)mine);
+}
+
+__global__ __launch_bounds__(kBlock) void lookup_kernel(const int64_t *__restrict__ positions,
+                                                        int64_t num, Lookup look) {
+  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (j < num) look(j, positions[j]);
+}
+
 struct SampleWs {
   size_t raw, ktmp, sorted, hist, total;
 };
@@ -271,5 +313,108 @@ extern "C" int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const
         sorted, num, trajectory_length, modulo, idxs, tss, lens);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
   }
+  return 0;
+}
+
+namespace gearhip {
+namespace {
+
+int check_lookup(const Lookup &look) {
+  if (look.index_n < 0 || look.lengths_n < 0) return GEAR_HIP_EINVAL;
+  if (look.lens && !look.lengths_table) return GEAR_HIP_EINVAL;
+  if (!look.sampled && !look.local && !look.lens) return GEAR_HIP_EINVAL;
+  return 0;
+}
+
+// raw: num positions on the device (each in [0, bound)); sorted ascending, then looked up.
+int sort_and_look_up(const int64_t *raw, int64_t num, int64_t bound, const Lookup &look, char *ws,
+                     const SampleWs &w, hipStream_t st) {
+  if (num <= radix::kRankMax && bound <= (1ll << 32)) {
+    rank_lookup_kernel<<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(
+        raw, (int)num, look);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  int key_bits = 1;
+  while (key_bits < 63 && ((uint64_t)(bound - 1) >> key_bits) != 0) ++key_bits;
+  int64_t *sorted = reinterpret_cast<int64_t *>(ws + w.sorted);
+  const int rc = radix::sort_pairs<uint64_t, uint64_t>(
+      reinterpret_cast<const uint64_t *>(raw), reinterpret_cast<uint64_t *>(sorted), nullptr,
+      nullptr, reinterpret_cast<uint64_t *>(ws + w.ktmp), nullptr, num, 0, key_bits,
+      reinterpret_cast<uint32_t *>(ws + w.hist), st);
+  if (rc) return rc;
+  lookup_kernel<<<dim3((unsigned)ceil_div64(num, kBlock)), dim3(kBlock), 0, st>>>(sorted, num, look);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return 0;
+}
+
+}  // namespace
+}  // namespace gearhip
+
+extern "C" int gear_hip_sample_lookup_f64(const double *prefix, int64_t n, const float *u,
+                                          int64_t num, int unit_uniforms,
+                                          const int64_t *index_table, int64_t index_offset,
+                                          const int64_t *lengths_table, int64_t lengths_n,
+                                          int64_t *sampled_out, int64_t *local_out,
+                                          int64_t *lens_out, void *workspace,
+                                          size_t workspace_bytes, void *stream) {
+  if (n < 0 || num < 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (n == 0 || !prefix || !u) return GEAR_HIP_EINVAL;
+  const Lookup look{index_table, n, index_offset, lengths_table, lengths_n, sampled_out, local_out,
+                    lens_out};
+  int rc = check_lookup(look);
+  if (rc) return rc;
+  const SampleWs w = sample_ws(num);
+  if (!workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 7))
+    return GEAR_HIP_EWORKSPACE;
+  const int64_t sblocks = ceil_div64(num, kSearchBlock);
+  if (sblocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  char *ws = static_cast<char *>(workspace);
+  int64_t *raw = reinterpret_cast<int64_t *>(ws + w.raw);
+  hipStream_t st = as_stream(stream);
+  search_f64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(
+      prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return sort_and_look_up(raw, num, n, look, ws, w, st);
+}
+
+extern "C" int gear_hip_sort_lookup_i64(const int64_t *positions, int64_t num, int64_t bound,
+                                        const int64_t *index_table, int64_t index_n,
+                                        int64_t index_offset, const int64_t *lengths_table,
+                                        int64_t lengths_n, int64_t *sampled_out,
+                                        int64_t *local_out, int64_t *lens_out, void *workspace,
+                                        size_t workspace_bytes, void *stream) {
+  if (num < 0 || bound <= 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (!positions) return GEAR_HIP_EINVAL;
+  const Lookup look{index_table, index_n, index_offset, lengths_table, lengths_n, sampled_out,
+                    local_out, lens_out};
+  int rc = check_lookup(look);
+  if (rc) return rc;
+  const SampleWs w = sample_ws(num);
+  if (!workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 7))
+    return GEAR_HIP_EWORKSPACE;
+  return sort_and_look_up(positions, num, bound, look, static_cast<char *>(workspace), w,
+                          as_stream(stream));
+}
+
+extern "C" int gear_hip_lookup_i64(const int64_t *positions, int64_t num,
+                                   const int64_t *index_table, int64_t index_n,
+                                   int64_t index_offset, const int64_t *lengths_table,
+                                   int64_t lengths_n, int64_t *sampled_out, int64_t *local_out,
+                                   int64_t *lens_out, void *stream) {
+  if (num < 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (!positions) return GEAR_HIP_EINVAL;
+  const Lookup look{index_table, index_n, index_offset, lengths_table, lengths_n, sampled_out,
+                    local_out, lens_out};
+  int rc = check_lookup(look);
+  if (rc) return rc;
+  const int64_t blocks = ceil_div64(num, kBlock);
+  if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  lookup_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream)>>>(positions, num,
+                                                                               look);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }

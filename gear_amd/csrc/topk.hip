@@ -51,16 +51,25 @@ constexpr int kBins0 = 16384;  // level-0 bins
 constexpr int kBinsR = 2048;   // bins of a refinement level (up to 11 bits)
 constexpr int kBinsF = 65536;  // bins of the two levels that run after a failed hint (16 bits)
 constexpr int kUniformShift = 18;  // level-0 bins without a sample: the top 14 bits of the key
-// with a sample: keys below the hint at 12 bits, a middle stretch up to the sample's top in up to
-// kMidBins bins of its own resolution, the rest above
-constexpr int kLowShift = 20, kMidBins = 10240, kMidBinsCoarse = 256;
+// with a sample: keys below the hint at 12 bits (numbered, never counted), a middle stretch up to
+// the sample's top in up to kMidBins (value order: even segments for the sort) or kMidBinsCoarse
+// bins of its own resolution, the rest above in at most kTopBins bins: at most kHintedBins bins
+// from the hint upwards, which are the ones that are counted
+constexpr int kLowShift = 20, kMidBins = 2048, kMidBinsCoarse = 256, kTopBins = 2046;
+constexpr int kHintedBins = 4096;
 // Keys of one level-0 bin differ in at most this many low bits, whichever stretch it lies in:
 // level 1 resolves the top 11 of them, level 2 the rest.
 constexpr int kMaxBinBits = 21;
 static_assert(kLowShift <= kMaxBinBits && kUniformShift <= kMaxBinBits, "coarse bins within the levels' reach");
-static_assert((1ll << (32 - kMaxBinBits)) <= kMidBins, "the middle stretch can always be cut finely enough");
-static_assert((1ll << 32 >> kLowShift) + kMidBins + (1ll << (32 - kMaxBinBits)) <= kBins0,
-              "the stretch above the largest sample keeps enough bins for bins of 2^kMaxBinBits keys");
+// (a stretch too wide for its bins at 2^kMaxBinBits keys apiece gets more of them: no more than
+// 2^11 + 3 for both stretches together when both are that wide.  1023 + 1022 bins, which would
+// let value order keep eight copies too, were measured: level 0 0.8 us faster, the sort 0.7 us
+// slower.)
+static_assert(kMidBins + 1 + kTopBins + 1 <= kHintedBins &&
+                  (1ll << (32 - kMaxBinBits)) + 3 <= kHintedBins &&
+                  (1ll << (32 - kMaxBinBits)) <= kMidBins && (1ll << (32 - kMaxBinBits)) <= kTopBins + 2,
+              "the bins from the hint upwards fit one copy of the histogram");
+static_assert((1ll << 32 >> kLowShift) + kHintedBins <= kBins0, "every bin has a number below kBins0");
 // The sample: 2, 8 or 32 priorities per thread of one workgroup (2048, 8192 or 32768).  One CU
 // sustains about one random miss per 1.2 ns, so the sample is as small as keeps the candidate
 // lists from overflowing: a loose bound lists too much, and after an overflow every later level
@@ -106,15 +115,13 @@ __device__ __forceinline__ uint32_t bin_hi_key(const BinMap &m, uint32_t bin) {
 }
 
 // The map around a hint: keys below a_end (a multiple of 2^kLowShift) in coarse bins, the stretch
-// a_end .. b_last in up to mid_bins bins of its own resolution, the keys above with what is left
-// of the kBins0 bins.  A bin never spans more than 2^kMaxBinBits keys -- the two levels below
-// resolve 11 and 10 bits --: a middle stretch too wide for mid_bins bins of that size gets more
-// of them, at most 2048, which the budget of kMidBins covers.
-// compact: the stretch above b_last is cut as coarsely as the levels below allow, so that the
-// bins from the hint upwards are few (at most 2050) and their histogram can be kept in several
-// copies (see Copies).
+// a_end .. b_last in up to mid_bins bins of its own resolution, the keys above in at most
+// kTopBins bins (top_coarse: as coarsely as the levels below allow).  A bin never spans more
+// than 2^kMaxBinBits keys -- the two levels below resolve 11 and 10 bits --: a stretch too wide
+// for its bins at that size gets more of them; the two stretches together then still stay below
+// 2^(32 - kMaxBinBits) + 3 bins.
 __device__ __forceinline__ BinMap make_map(uint32_t a_end, uint32_t b_last, int mid_bins,
-                                           bool compact) {
+                                           bool top_coarse) {
   BinMap map;
   map.uniform = 0u;
   map.a_end = a_end;
@@ -126,18 +133,20 @@ __device__ __forceinline__ BinMap make_map(uint32_t a_end, uint32_t b_last, int 
   map.nb0 = map.a_end >> kLowShift;
   map.nc0 = map.nb0 + (span >> map.b_shift) + 1u;
   const uint32_t rest = 0xffffffffu - map.b_last;  // keys above the middle stretch
-  while (rest != 0u && map.nc0 + ((rest - 1u) >> map.c_shift) >= (uint32_t)kBins0) ++map.c_shift;
-  if (compact && rest != 0u) map.c_shift = (uint32_t)kMaxBinBits;
+  while (rest != 0u && map.c_shift < (uint32_t)kMaxBinBits &&
+         ((rest - 1u) >> map.c_shift) >= (uint32_t)kTopBins)
+    ++map.c_shift;
+  if (top_coarse && rest != 0u) map.c_shift = (uint32_t)kMaxBinBits;
   return map;
 }
 
-// The level-0 histogram of the candidates in several copies.  Every workgroup of level 0 adds
+// The level-0 histogram of a map with a hint holds the bins from the hint upwards only (at most
+// kHintedBins; bin b is counted at b - nb0), in several copies.  Every workgroup of level 0 adds
 // its counts to the histogram in memory at the end, all of them at about the same time and to
-// the same few cache lines, and atomics on one line are served one after the other (about 16 ns
-// apiece: 245 workgroups, 4 us).  Where the places in value order of the bins are not asked for
-// (the index-ordered selection, large k) the bins from the hint upwards are few -- a compact
-// map --, the histogram is kept in 8 copies (4 when it has more than 2048 bins), workgroup b adds
-// to copy b mod 8, and level 1 adds the copies up when it picks: 3 us less for level 0.
+// the same cache lines, and atomics on one line are served one after the other (about 16 ns
+// apiece: 245 workgroups, 4 us; more with more lines).  With 8 copies (4 when the histogram has
+// more than 2048 bins: value order) workgroup b adds to copy b mod 8, and level 1 adds the
+// copies up when it picks: 3 us less for level 0.
 struct Copies {
   uint32_t used;    // bins from the hint upwards: bin b is counted at b - nb0
   uint32_t copies;  // 8 or 4
@@ -148,7 +157,7 @@ __device__ __forceinline__ Copies copies_of(const BinMap &m) {
   const uint32_t rest = 0xffffffffu - m.b_last;
   c.used = (m.nc0 - m.nb0) + (rest != 0u ? ((rest - 1u) >> m.c_shift) + 1u : 0u);
   c.copies = c.used <= (uint32_t)kBins0 / 8u ? 8u : 4u;
-  c.pitch = (uint32_t)kBins0 / c.copies;
+  c.pitch = (uint32_t)kBins0 / c.copies;  // (used <= kHintedBins = kBins0 / 4)
   return c;
 }
 
@@ -176,7 +185,8 @@ struct State {
   // the mark of a call with the same n, k and bin resolution
   uint64_t next_magic;
   uint32_t next_a_end, next_b_last;
-  uint32_t pad[40];
+  uint32_t low_seg;  // after a failed hint, value order: the segment of the entries below the hint
+  uint32_t pad[39];
 };
 static_assert(sizeof(State) == 256, "State is the 256-byte header of the workspace");
 
@@ -670,14 +680,13 @@ __device__ __forceinline__ uint32_t lanes_before(uint64_t mask, uint32_t acc) {
                                    __builtin_amdgcn_mbcnt_lo((uint32_t)mask, acc));
 }
 
-template <bool COMPACT>  // the histogram holds the bins from the hint upwards only, in copies
 __global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
     const float *__restrict__ p, int64_t n, const State *state, uint32_t *__restrict__ hist0,
     int64_t wave_len, uint32_t *__restrict__ wave_listed, uint64_t *__restrict__ lists,
     int list_cap) {
-  __shared__ __align__(16) uint32_t h[kBins0];
+  __shared__ __align__(16) uint32_t h[kHintedBins];  // the bins from the hint upwards
   __shared__ uint64_t queue[kWavesPerBlock][kQueueCap];
-  __shared__ uint32_t s_touched[kBins0 / kWave];  // runs of 64 bins that hold a count
+  __shared__ uint32_t s_touched[kHintedBins / kWave];  // runs of 64 bins that hold a count
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   const int64_t begin = gw * wave_len;
@@ -698,12 +707,12 @@ __global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
 #pragma unroll
     for (int a = 0; a < kAhead; ++a) load_step(a, qa[a]);
   }
-  for (int i = tid * 4; i < kBins0; i += kThreads * 4)
-    *reinterpret_cast<u32x4 *>(&h[i]) = u32x4{0u, 0u, 0u, 0u};
-  if (tid < kBins0 / kWave) s_touched[tid] = 0u;
+  static_assert(kHintedBins == kThreads * 4, "one 16-byte store per thread clears the histogram");
+  *reinterpret_cast<u32x4 *>(&h[tid * 4]) = u32x4{0u, 0u, 0u, 0u};
+  if (tid < kHintedBins / kWave) s_touched[tid] = 0u;
   const BinMap map = state->map;
   const float lo_f = lower_bound_float(map.a_end);
-  const uint32_t bin_base = COMPACT ? map.nb0 : 0u;  // candidates' bins are counted from here
+  const uint32_t bin_base = map.nb0;  // candidates' bins are counted from here
   const uint32_t cap = (uint32_t)(list_cap < kQueueCap ? list_cap : kQueueCap);
   const uint32_t first_index = (uint32_t)begin + (uint32_t)lane * 4u;
   uint64_t *wq = queue[wave];
@@ -794,14 +803,11 @@ __global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
   // any: atomics of a wave that fall into one cache line travel as one request, and requests to
   // a line are served one after the other -- candidates that each added their own bin's count
   // sent some 50 000 requests to the eight lines of 256 coarse bins, 20 to 35 us.  Wave w looks
-  // after the runs w, w + 16, ...
-  static_assert(kBins0 / kWave == kWavesPerBlock * 16, "sixteen runs of bins per wave");
-  uint32_t *mine = hist0;
-  if (COMPACT) {
-    const Copies cp = copies_of(map);
-    mine += (blockIdx.x % cp.copies) * cp.pitch;
-  }
-  const uint32_t flag = lane < 16 ? s_touched[wave + kWavesPerBlock * lane] : 0u;
+  // after the runs w, w + 16, w + 32 and w + 48, in this workgroup's copy of the histogram.
+  static_assert(kHintedBins / kWave == kWavesPerBlock * 4, "four runs of bins per wave");
+  const Copies cp = copies_of(map);
+  uint32_t *mine = hist0 + (blockIdx.x % cp.copies) * cp.pitch;
+  const uint32_t flag = lane < 4 ? s_touched[wave + kWavesPerBlock * lane] : 0u;
   for (uint64_t todo = wave_ballot(flag != 0u); todo != 0ull; todo &= todo - 1ull) {
     const int run = wave + kWavesPerBlock * (__ffsll((unsigned long long)todo) - 1);
     const uint32_t c = h[run * kWave + lane];
@@ -849,28 +855,36 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
     if (h[i]) atomicAdd(&hist0[i], h[i]);
 }
 
-// pick_bin for the level-0 histogram of a compact map (see Copies): the bins from the hint
-// upwards, at most 4096, kept in several copies that are added up here.  Returns the picked bin
-// under its number in the map.  Every thread of the workgroup calls.
+// pick_bin for the level-0 histogram of a map with a hint (see Copies): the bins from the hint
+// upwards, at most kHintedBins, kept in several copies that are added up here into `sums` (LDS,
+// kHintedBins words).  Returns the picked bin under its number in the map; boff, wg_bins and
+// seg_shift as for pick_bin.  Every thread of the workgroup calls.
 __device__ __forceinline__ Pick pick_copies(uint32_t k_rem, const uint32_t *hist, const BinMap &map,
-                                            uint32_t rank2, uint32_t *bin2) {
+                                            uint32_t rank2, uint32_t *bin2, uint32_t *sums,
+                                            uint32_t *boff, uint32_t *wg_bins, int seg_shift) {
   constexpr int kPer = 4;  // bins per thread, top down: thread 0 owns the top four
-  static_assert(kPer * kThreads * 4 == kBins0, "a copy of up to 4096 bins");
+  static_assert(kPer * kThreads == kHintedBins, "every bin of a copy has its thread");
   __shared__ uint32_t wsum[kWavesPerBlock];
   __shared__ Pick s_pick;
   __shared__ uint32_t s_bin2;
+  __shared__ uint32_t s_base[kHintedBins / kWave];  // entries above every 64th bin from the top
   const Copies cp = copies_of(map);
   const int tid = threadIdx.x, lane = tid & 63;
+  // the copies are added up into `sums` (LDS, 4096 words): neighbouring threads take neighbouring
+  // bins, and a thread's loads of the copies of its bin are all under way together
+  for (uint32_t at = (uint32_t)tid; at < cp.used; at += kThreads) {
+    uint32_t v[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = (uint32_t)r < cp.copies ? hist[(uint32_t)r * cp.pitch + at] : 0u;
+    sums[at] = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+  }
+  __syncthreads();
   uint32_t c[kPer];
   uint32_t tsum = 0u;
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
     const uint32_t from_top = (uint32_t)(tid * kPer + j);
-    c[j] = 0u;
-    if (from_top < cp.used) {
-      const uint32_t at = cp.used - 1u - from_top;
-      for (uint32_t r = 0; r < cp.copies; ++r) c[j] += hist[r * cp.pitch + at];
-    }
+    c[j] = from_top < cp.used ? sums[cp.used - 1u - from_top] : 0u;
     tsum += c[j];
   }
   const int inc = wave_inclusive_sum((int)tsum);
@@ -907,7 +921,43 @@ __device__ __forceinline__ Pick pick_copies(uint32_t k_rem, const uint32_t *hist
   find(k_rem, &s_pick.bin, &s_pick.k_rem);
   if (rank2 != 0u) find(rank2, &s_bin2, nullptr);
   if (tid == kThreads - 1) s_pick.total = running0 + tsum;
+  if (boff && (tid * kPer) % kWave == 0) s_base[tid * kPer / kWave] = running0;
   __syncthreads();
+  // Where the bins at or above the picked one start in value order, and the segment table: as
+  // in pick_bin (the workgroups of the launch share the bins in runs of 64, a bin per lane),
+  // with the counts taken from the sums in LDS.
+  if (boff) {
+    const uint32_t used = cp.used;
+    const int per = (int)((((used + gridDim.x - 1u) / gridDim.x) + kWave - 1u) & ~(uint32_t)(kWave - 1));
+    const int r_begin = (int)blockIdx.x * per;
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    const uint64_t gt_mask = lane == 63 ? 0ull : (~0ull << (lane + 1));
+    for (int ch = tid >> 6; ch * kWave < per && r_begin + ch * kWave < (int)used; ch += kWavesPerBlock) {
+      const int r = r_begin + ch * kWave + lane;  // the bin's rank from the top
+      const bool real = r < (int)used;
+      const uint32_t bin = map.nb0 + used - 1u - (uint32_t)(real ? r : 0);
+      const uint32_t cnt = real ? sums[used - 1u - (uint32_t)r] : 0u;
+      const uint32_t inc_b = (uint32_t)wave_inclusive_sum((int)cnt);
+      const uint32_t above = s_base[(r_begin + ch * kWave) / kWave] + inc_b - cnt;
+      const bool sel = real && above < k_rem;
+      if (sel) boff[bin] = above;
+      const bool ne = sel && cnt != 0u;
+      const uint32_t w = above >> seg_shift;
+      const uint64_t nem = wave_ballot(ne);
+      const uint64_t lower = nem & lt_mask, upper = nem & gt_mask;
+      const int prev = lower ? 63 - __builtin_clzll(lower) : lane;
+      const int next = upper ? __builtin_ctzll(upper) : lane;
+      const uint32_t w_prev = (uint32_t)__shfl((int)w, prev), w_next = (uint32_t)__shfl((int)w, next);
+      if (ne && (lower == 0ull || w_prev != w)) {
+        atomicMax(&wg_bins[4 * w], bin + 1u);
+        atomicMax(&wg_bins[4 * w + 2], ~above);
+      }
+      if (ne && (upper == 0ull || w_next != w)) {
+        atomicMax(&wg_bins[4 * w + 1], (uint32_t)kBins0 - bin);
+        atomicMax(&wg_bins[4 * w + 3], above + cnt);
+      }
+    }
+  }
   if (bin2) *bin2 = s_bin2;
   return s_pick;
 }
@@ -1015,7 +1065,8 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
     const uint64_t *__restrict__ lists, int list_cap) {
   __shared__ uint32_t hp[kBinsF / 2];  // packed counters after a failed hint; else h, below
   uint32_t *h = hp;
-  static_assert(kBinsR <= kBinsF / 2, "the level's histogram fits the same LDS");
+  static_assert(kBinsR + kHintedBins <= kBinsF / 2,
+                "the level's histogram and the sums of the level-0 copies fit the same LDS");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int i = tid; i < kBinsR; i += kThreads) h[i] = 0u;
   // the wave's list does not depend on the pick: its length and first stretch are asked for
@@ -1038,11 +1089,11 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
     const bool hinted = map.uniform == 0u && hint_bin != kNoLists;
     // (the 2k-th largest key, where the histogram holds that many: the next call's hint)
     uint32_t bin2 = 0u;
-    // (a hinted call that does not ask for the bins' places in value order has a compact map)
-    const bool compact = hinted && boff == nullptr;
-    const Pick r = compact ? pick_copies((uint32_t)k, hist_prev, map, 2u * (uint32_t)k, &bin2)
-                           : pick_bin<kBins0>((uint32_t)k, hist_prev, boff, wg_bins, seg_shift,
-                                              hinted ? 2u * (uint32_t)k : 0u, &bin2);
+    // (with a hint the histogram holds the bins from the hint upwards, in copies, which are added
+    // up in the part of the LDS that only a failed hint uses, later)
+    const Pick r = hinted ? pick_copies((uint32_t)k, hist_prev, map, 2u * (uint32_t)k, &bin2,
+                                        hp + kBinsR, boff, wg_bins, seg_shift)
+                          : pick_bin<kBins0>((uint32_t)k, hist_prev, boff, wg_bins, seg_shift);
     fail = hinted && r.found == 0u;
     lo = bin_lo_key(map, r.bin);
     hi = bin_hi_key(map, r.bin);
@@ -1068,11 +1119,11 @@ __global__ __launch_bounds__(kThreads) void member_hist_kernel(
       }
       if (fail && boff != nullptr) {
         // Value order: the entries below the hint that end up selected follow the r.total
-        // candidates in the output.  Every coarse bin below the hint got boff = r.total above
-        // (all of them lie "above the k-th"), so those entries go to the segment in whose
-        // stretch place r.total lies; that segment's table entry is widened to the coarse bins
-        // [0, nb0) and to the rest of the output.
+        // candidates in the output.  They go to the segment in whose stretch of the output place
+        // r.total lies (write finds it in the state); that segment's table entry is widened to
+        // the coarse bins [0, nb0) and to the rest of the output.
         const uint32_t w = r.total >> seg_shift;
+        state->low_seg = w;
         atomicMax(&wg_bins[4 * w], map.nb0);
         atomicMax(&wg_bins[4 * w + 1], (uint32_t)kBins0);
         atomicMax(&wg_bins[4 * w + 2], ~r.total);
@@ -1256,6 +1307,8 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
   const uint32_t need_eq = state->k_rem[2];
   const bool reread = m_raw == kListFull;
   const BinMap map = state->map;
+  const uint32_t low_seg = state->low_seg;
+  const uint32_t low_end = state->fail != 0u ? map.a_end : 0u;  // keys below: under a failed hint
 
   // counts of the workgroups before this one (at most kMaxBlocks), then of the waves before
   // this one in its own workgroup
@@ -1303,7 +1356,9 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
         cidx[pos] = index;
         // the segment of the sort that takes the entry: the one in whose stretch of the
         // output the entry's level-0 bin starts (ties at T belong to none)
-        cseg[pos] = is_eq ? (uint8_t)kNoSegment : (uint8_t)(boff[bin_of(map, key)] >> seg_shift);
+        // (entries below a failed hint have no counted bin: their segment is in the state)
+        cseg[pos] = is_eq ? (uint8_t)kNoSegment
+                          : (uint8_t)(key < low_end ? low_seg : boff[bin_of(map, key)] >> seg_shift);
       }
     }
   };
@@ -2010,8 +2065,8 @@ int topk_launch(const float *priorities, int64_t n, int64_t k, int sorted_by_val
   const int64_t zero_words = (int64_t)((l.zero_end - l.zero_begin) / 4);
   const unsigned zero_blocks = (unsigned)ceil_div64(zero_words, (int64_t)kThreads * 4);
   const dim3 block(kThreads), grid((unsigned)g.blocks);
-  // Fine bins pay off in the value-order sort (small, even segments) but cost level 0 an atomic
-  // per candidate when its histogram is flushed; the index-ordered selection takes coarse ones.
+  // Finer bins pay off in the value-order sort (small, even segments) but cost level 0 more
+  // cache lines to add its counts to; the index-ordered selection takes coarse ones.
   const int mid_bins = (sorted_by_value && k <= kBucketMaxK) ? kMidBins : kMidBinsCoarse;
   {
     uint32_t *zero = reinterpret_cast<uint32_t *>(ws + l.zero_begin);
@@ -2026,12 +2081,9 @@ int topk_launch(const float *priorities, int64_t n, int64_t k, int sorted_by_val
       prep_kernel<32><<<pgrid, block, 0, st>>>(priorities, n, k, rank, list_all, mid_bins, warm, state,
                                                zero, zero_words);
   }
-  if (rank != 0u && mid_bins == kMidBinsCoarse)
-    level0_hinted_kernel<true><<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len,
-                                                       wave_listed, lists, (int)g.list_cap);
-  else if (rank != 0u)
-    level0_hinted_kernel<false><<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len,
-                                                        wave_listed, lists, (int)g.list_cap);
+  if (rank != 0u)
+    level0_hinted_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len,
+                                                 wave_listed, lists, (int)g.list_cap);
   else
     level0_kernel<<<grid, block, 0, st>>>(priorities, n, state, hist0, g.wave_len, wave_listed,
                                           lists, (int)g.list_cap);

@@ -108,6 +108,7 @@ class OfflineLoader(BasicLoader):
         self._indices = torch.arange(self._iset.local_capacity, dtype=torch.long,
                                      device=self._mpu.device) + self._iset.index_offset
         self.last_masks = None
+        self.last_sampled = None   # global indices of the last batch (device tensor)
 
     def refresh_index(self):
         """Upload priorities and trajectory lengths after the host side changed them."""
@@ -218,11 +219,31 @@ class OfflineLoader(BasicLoader):
         self.last_masks = masks
         return data_batch
 
+    def _select_gather(self, draws, dirty_from):
+        """Everything of a step after the draws: the sampler's own preparation (prefix rescan,
+        top-k selection), then ONE call that sorts the batch, looks up global index, local index
+        and recorded length of every entry, and gathers all columns
+        (CpuTrajectoryStorageHandler.select_subcopy).  Returns (sampled, lengths, data_batch)."""
+        kind, picks, prefix = self._sampler.prepare(self._indices, self._device_weights, draws,
+                                                    dirty_from=dirty_from)
+        n = picks.numel()
+        dev = self._mpu.device
+        looked = torch.empty((3, n), dtype=torch.int64, device=dev)  # sampled, local, lengths
+        data_batch = self._empty_batch(n)
+        masks = None
+        if self._with_mask:
+            masks = [torch.empty((n, p.length), dtype=torch.uint8, device=dev)
+                     for p in self._patterns]
+        self._handler.select_subcopy(kind, picks, prefix, self._indices, self._iset.index_offset,
+                                     self._device_timesteps, self._sub_cols, data_batch, True,
+                                     masks, looked[0], looked[1], looked[2])
+        self.last_masks = masks
+        self.last_sampled = looked[0]
+        return looked[0], looked[2], data_batch
+
     def _graph_step(self):
-        sampled = self._sampler.select(self._indices, self._device_weights, self._graph_draws)
-        local = sampled - self._iset.index_offset if self._iset.index_offset else sampled
-        lengths = ops.take_i64(self._device_timesteps, local)
-        return lengths, self._gather(local, lengths)
+        _, lengths, data_batch = self._select_gather(self._graph_draws, None)
+        return lengths, data_batch
 
     def _graph_iterate(self):
         n = self._indices.numel()
@@ -251,15 +272,9 @@ class OfflineLoader(BasicLoader):
     def fused_iterate(self):
         if self._use_graph:
             return self._graph_iterate()
-        sampled = self._sampler.sync_sample(self._indices, self._device_weights,
-                                            self._batch_size * self._dp_world,
-                                            dirty_from=self._dirty_from)
+        draws = self._sampler.draw(self._indices.numel(), self._batch_size * self._dp_world)
+        _, lengths, data_batch = self._select_gather(draws, self._dirty_from)
         self._dirty_from = self._device_weights.numel()   # clean until the next update
-        local = sampled
-        if self._iset.index_offset:
-            local = sampled - self._iset.index_offset
-        lengths = ops.take_i64(self._device_timesteps, local)
-        data_batch = self._gather(local, lengths)
         timesteps = lengths if self._timesteps_on_device else lengths.cpu()
         return timesteps, data_batch
 

@@ -146,6 +146,52 @@ def subcopy_multi(src, idxs, tss, lens, traj_stride, columns, capacity=0, trajec
          int(traj_stride), int(capacity), int(trajectory_length), descs, n, _stream())
 
 
+class GatherPlan:
+    """subcopy_multi for a loop that gathers into the same batch tensors every step: the column
+    descriptors and every argument that does not change are marshalled once, run() is one call
+    into the library with the three index tensors of the step."""
+
+    def __init__(self, src, traj_stride, columns, num, capacity=0, trajectory_length=0):
+        n = len(columns)
+        if n > _cabi.MAX_COLUMNS:
+            raise ValueError("at most %d columns per launch" % _cabi.MAX_COLUMNS)
+        self._descs = (ColumnDesc * max(n, 1))()
+        self._keep = []
+        for i, c in enumerate(columns):
+            dst = c["dst"]
+            stride = c.get("dst_stride", c["span"] * c["step_bytes"])
+            if not dst.is_cuda or not dst.is_contiguous():
+                raise ValueError("column %d: dst must be a contiguous GPU tensor" % i)
+            if dst.numel() * dst.element_size() < num * stride:
+                raise ValueError("column %d: dst is smaller than num * dst_stride bytes" % i)
+            m = c.get("mask_out")
+            if m is not None and m.numel() < num * c["span"]:
+                raise ValueError("column %d: mask_out is smaller than num * span" % i)
+            d = self._descs[i]
+            d.dst = dst.data_ptr()
+            d.mask_out = m.data_ptr() if m is not None else None
+            d.ofst, d.span = int(c["ofst"]), int(c["span"])
+            d.step_bytes, d.col_base, d.dst_stride = int(c["step_bytes"]), int(c["col_base"]), int(stride)
+            d.pad_head = int(bool(c["pad_head"]))
+            d.zero_fill = int(bool(c.get("zero_fill", True)))
+            self._keep.append((dst, m))
+        self._keep.append(src)
+        self._fn = load().gear_hip_subcopy_multi_checked
+        self._num = int(num)
+        self._head = (_src_ptr(src), self._num)
+        self._tail = (int(traj_stride), int(capacity), int(trajectory_length), self._descs, n)
+
+    def run(self, idxs, tss, lens):
+        if idxs.numel() != self._num or tss.numel() != self._num or lens.numel() != self._num:
+            raise ValueError("the plan was made for %d windows" % self._num)
+        if idxs.dtype != torch.int64 or tss.dtype != torch.int64 or lens.dtype != torch.int64:
+            raise TypeError("idxs, tss and lens must be int64 tensors")
+        code = self._fn(*self._head, idxs.data_ptr(), tss.data_ptr(), lens.data_ptr(), *self._tail,
+                        _stream_value(idxs.device))
+        if code != 0:
+            _cabi.check("gear_hip_subcopy_multi_checked", code)
+
+
 def vcopy(src, dst, src_offsets, dst_offsets, strides, max_stride):
     _need(src_offsets, torch.int64, "src_offsets")
     _need(dst_offsets, torch.int64, "dst_offsets")
@@ -343,6 +389,74 @@ def sample_sorted(prefix, u, *, unit_uniforms=True, sorted_out=None, trajectory_
     if trajectory_length > 0:
         return sorted_out, idxs, tss, lens
     return sorted_out
+
+
+def _lookup_outputs(num, dev, lengths_table, sampled_out, local_out, lens_out):
+    empty = lambda: torch.empty(num, dtype=torch.int64, device=dev)
+    sampled = sampled_out if sampled_out is not None else empty()
+    local = local_out if local_out is not None else empty()
+    lens = lens_out if lens_out is not None else (empty() if lengths_table is not None else None)
+    return sampled, local, lens
+
+
+def sample_lookup(prefix, u, *, unit_uniforms=True, index_table=None, index_offset=0,
+                  lengths_table=None, sampled_out=None, local_out=None, lens_out=None):
+    """Weighted draws, sorted, with the loader's look-ups in the same call: positions of the
+    draws in the fp64 prefix, ascending -> (sampled = index_table[position], local = sampled -
+    index_offset, lens = lengths_table[local]).  See gear_hip_sample_lookup_f64."""
+    _need(prefix, torch.float64, "prefix")
+    _need(u, torch.float32, "u")
+    num, dev = u.numel(), u.device
+    if index_table is not None:
+        _need(index_table, torch.int64, "index_table")
+        if index_table.numel() != prefix.numel():
+            raise ValueError("index_table and prefix differ in length")
+    if lengths_table is not None:
+        _need(lengths_table, torch.int64, "lengths_table")
+    sampled, local, lens = _lookup_outputs(num, dev, lengths_table, sampled_out, local_out, lens_out)
+    ws = _ws.get("sample", load().gear_hip_sample_workspace_bytes(num), dev)
+    call("gear_hip_sample_lookup_f64", _ptr(prefix), prefix.numel(), _ptr(u), num,
+         int(bool(unit_uniforms)), _ptr(index_table), int(index_offset), _ptr(lengths_table),
+         lengths_table.numel() if lengths_table is not None else 0, _ptr(sampled), _ptr(local),
+         _ptr(lens), _ptr(ws), ws.numel(), _stream())
+    return sampled, local, lens
+
+
+def sort_lookup(positions, bound, *, index_table=None, index_offset=0, lengths_table=None,
+                sampled_out=None, local_out=None, lens_out=None):
+    """Given positions (each in [0, bound)): ascending sort, then the same look-ups
+    (gear_hip_sort_lookup_i64)."""
+    _need(positions, torch.int64, "positions")
+    num, dev = positions.numel(), positions.device
+    if index_table is not None:
+        _need(index_table, torch.int64, "index_table")
+    if lengths_table is not None:
+        _need(lengths_table, torch.int64, "lengths_table")
+    sampled, local, lens = _lookup_outputs(num, dev, lengths_table, sampled_out, local_out, lens_out)
+    ws = _ws.get("sample", load().gear_hip_sample_workspace_bytes(num), dev)
+    call("gear_hip_sort_lookup_i64", _ptr(positions), num, int(bound), _ptr(index_table),
+         index_table.numel() if index_table is not None else 0, int(index_offset),
+         _ptr(lengths_table), lengths_table.numel() if lengths_table is not None else 0,
+         _ptr(sampled), _ptr(local), _ptr(lens), _ptr(ws), ws.numel(), _stream())
+    return sampled, local, lens
+
+
+def lookup(positions, *, index_table=None, index_offset=0, lengths_table=None, sampled_out=None,
+           local_out=None, lens_out=None):
+    """The look-ups alone, for positions that are already in the wanted order
+    (gear_hip_lookup_i64)."""
+    _need(positions, torch.int64, "positions")
+    num, dev = positions.numel(), positions.device
+    if index_table is not None:
+        _need(index_table, torch.int64, "index_table")
+    if lengths_table is not None:
+        _need(lengths_table, torch.int64, "lengths_table")
+    sampled, local, lens = _lookup_outputs(num, dev, lengths_table, sampled_out, local_out, lens_out)
+    call("gear_hip_lookup_i64", _ptr(positions), num, _ptr(index_table),
+         index_table.numel() if index_table is not None else 0, int(index_offset),
+         _ptr(lengths_table), lengths_table.numel() if lengths_table is not None else 0,
+         _ptr(sampled), _ptr(local), _ptr(lens), _stream())
+    return sampled, local, lens
 
 
 def upper_bound_i64(prefix, u, *, unit_uniforms=True, idx_out=None):

@@ -63,6 +63,13 @@ class UniformSampler:
     def select(self, indices, weights, draws, dirty_from=None):
         return self._take_sorted(indices, draws)
 
+    # For a loader that hands the rest of its step to ONE library call
+    # (CpuTrajectoryStorageHandler.select_subcopy): what is left of select() before the sort and
+    # the look-ups, as (kind, positions-or-draws, prefix-or-None).  Only valid where
+    # indices_ascending holds.
+    def prepare(self, indices, weights, draws, dirty_from=None):
+        return "uniform", draws, None
+
     def _dp_rank_zero_sync(self, indices, weights, batch_size, dirty_from=None):
         device = self._mpu.device
         indices = ensure_tensor(indices, device, torch.int64)
@@ -95,6 +102,10 @@ class WeightedSampler(UniformSampler):
         self.last_positions = positions
         return self._take_sorted(indices, positions, positions_sorted=True)
 
+    def prepare(self, indices, weights, draws, dirty_from=None):
+        self._prefix = self._state.scan(weights, 0 if dirty_from is None else int(dirty_from))
+        return "weighted", draws, self._prefix
+
     def sample_with_importance(self, indices, weights, batch_size, beta=0.4):
         """Draw a batch and its importance weights (N * P(i)) ** -beta / max over the batch.
         Returns (indices, is_weights) in draw order (not sorted), aligned element by element."""
@@ -116,5 +127,17 @@ class TopKSampler(UniformSampler):
         return torch.empty(batch_size, dtype=torch.int64, device=self._mpu.device)  # size only
 
     def select(self, indices, weights, draws, dirty_from=None):
-        _, positions = ops.topk(weights, draws.numel(), sorted_by_value=False, want_values=False)
+        # the selection is repeated on an array that changes a little between batches: every
+        # call after the first takes up the bound the call before it left (same result)
+        if getattr(self, "_topk_state", None) is None:
+            self._topk_state = ops.TopKState()
+        _, positions = self._topk_state.select(weights, draws.numel(), sorted_by_value=False,
+                                               want_values=False)
         return self._take_sorted(indices, positions, positions_sorted=True)  # index-ordered
+
+    def prepare(self, indices, weights, draws, dirty_from=None):
+        if getattr(self, "_topk_state", None) is None:
+            self._topk_state = ops.TopKState()
+        _, positions = self._topk_state.select(weights, draws.numel(), sorted_by_value=False,
+                                               want_values=False)
+        return "positions", positions, None

@@ -286,6 +286,41 @@ int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const float *u, 
                                int64_t modulo, int64_t *idxs, int64_t *tss, int64_t *lens,
                                void *workspace, size_t workspace_bytes, void *stream);
 
+/* Batch selection with the look-ups the loader performs before it can gather, in one call.
+ * For a batch of positions into the loader's index array, sorted ascending, the entry at sorted
+ * place r with position p yields
+ *     sampled_out[r] = index_table ? index_table[p] : p      (0 for p outside [0, index_n))
+ *     local_out[r]   = sampled_out[r] - index_offset
+ *     lens_out[r]    = lengths_table[local_out[r]]            (0 outside [0, lengths_n))
+ * Any of the three outputs may be NULL (not all); lens_out needs lengths_table.  This replaces,
+ * for a sampler whose index array ascends (then sort(indices[p]) == indices[sort(p)]), the chain
+ * torch.sort(concat_indices[draws]) (gear/sampler/global_sampler.py:131,172,196),
+ * indices - index_offset and iset.timesteps[indices.cpu()] on the host
+ * (gear/loader/offline_loader.py:161-177): up to 4096 positions take ONE launch after the search
+ * (the ranking sort does the look-ups of the entry it places), more take the radix sort and an
+ * element-wise launch.
+ *   gear_hip_sample_lookup_f64  positions = upper_bound of the draws u in the fp64 prefix, as
+ *                               gear_hip_upper_bound_f64 (index_table, when given, has n entries)
+ *   gear_hip_sort_lookup_i64    positions given (uniform draws), each in [0, bound)
+ *   gear_hip_lookup_i64         positions given and already in the wanted order (the top-k's
+ *                               index-ordered selection): look-ups only, no workspace
+ * workspace: gear_hip_sample_workspace_bytes(num) bytes on the device. */
+int gear_hip_sample_lookup_f64(const double *prefix, int64_t n, const float *u, int64_t num,
+                               int unit_uniforms, const int64_t *index_table,
+                               int64_t index_offset, const int64_t *lengths_table,
+                               int64_t lengths_n, int64_t *sampled_out, int64_t *local_out,
+                               int64_t *lens_out, void *workspace, size_t workspace_bytes,
+                               void *stream);
+int gear_hip_sort_lookup_i64(const int64_t *positions, int64_t num, int64_t bound,
+                             const int64_t *index_table, int64_t index_n, int64_t index_offset,
+                             const int64_t *lengths_table, int64_t lengths_n,
+                             int64_t *sampled_out, int64_t *local_out, int64_t *lens_out,
+                             void *workspace, size_t workspace_bytes, void *stream);
+int gear_hip_lookup_i64(const int64_t *positions, int64_t num, const int64_t *index_table,
+                        int64_t index_n, int64_t index_offset, const int64_t *lengths_table,
+                        int64_t lengths_n, int64_t *sampled_out, int64_t *local_out,
+                        int64_t *lens_out, void *stream);
+
 /* Same search in an int64 prefix array (exact): t_j = floor(u[j] * prefix[n-1]) with u fp64 in
  * [0,1) when unit_uniforms != 0, else t_j = (int64) u[j] taken from an int64 array passed
  * through `u` (cast).  idx_out[j] = min(#{i : prefix[i] <= t_j}, n-1). */

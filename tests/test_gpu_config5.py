@@ -73,6 +73,7 @@ def test_config5_workload_three_steps_against_the_oracle(oracle):
         cols = [dict(dst=dsts[c], ofst=OFST, span=SPAN, step_bytes=STEP_BYTES[c],
                      col_base=int(accu[c]) * T, pad_head=True, zero_fill=True) for c in range(4)]
         near_edge = 0
+        selection = ops.TopKState()      # steps after the first start from the last step's bound
         for step in range(3):
             upd_idx = rng.permutation(NPRI)[:M].astype(np.int64)        # unique indices
             upd_val = (rng.lognormal(0, 1, size=M) ** 0.6).astype(np.float32)
@@ -82,7 +83,7 @@ def test_config5_workload_three_steps_against_the_oracle(oracle):
             announce("config 5 step %d: scatter -> top-k -> rescan -> draw -> host-table gather" % step)
             ops.scatter(pri, torch.from_numpy(upd_idx).cuda(), torch.from_numpy(upd_val).cuda(),
                         unique_indices=True)
-            vals, tidx = ops.topk(pri, K, sorted_by_value=True)
+            vals, tidx = selection.select(pri, K, sorted_by_value=True)
             ops.prefix_sum(pri, out=prefix)
             flat, idxs, tss, lens = ops.sample_sorted(prefix, torch.from_numpy(u01).cuda(),
                                                       unit_uniforms=True, trajectory_length=T,
@@ -126,6 +127,70 @@ def test_config5_workload_three_steps_against_the_oracle(oracle):
                                         STEP_BYTES[c], int(accu[c]) * T, threads=8)
                 assert np.array_equal(dsts[c].cpu().numpy(), exp), "step %d column %d" % (step, c)
         assert near_edge <= 1                             # < 1e-6 of draws in any realistic run
+    finally:
+        torch.cuda.synchronize()
+        assert lib.gear_hip_host_free(host_ptr) == 0
+
+
+def test_config5_full_size_host_table_window_by_window():
+    """Config 5's table at its full size: 2 000 trajectories x 1000 steps of the Atari schema,
+    56.5 GB of pinned, mapped host memory, filled from a seeded device generator.  2048 windows
+    drawn by priority over the 2 000 000 steps are gathered, all four columns, through the device
+    alias of the host pointer (offsets far beyond 32 bits), and every window is compared with
+    numpy slicing of the SAME host memory.  Skipped with the reason where the box cannot pin that
+    much."""
+    from gear_amd import _cabi, ops
+    lib = _cabi.load()
+    cap = 2000
+    row = sum(STEP_BYTES)
+    S = row * T
+    nbytes = S * cap
+    accu = np.concatenate([[0], np.cumsum(STEP_BYTES)])
+    host_ptr, dev_ptr = ctypes.c_void_p(), ctypes.c_void_p()
+    announce("config 5 full size: pinning a %.1f GB host table" % (nbytes / 1e9))
+    rc = lib.gear_hip_host_alloc(nbytes, ctypes.byref(host_ptr), ctypes.byref(dev_ptr))
+    if rc != 0:
+        pytest.skip("this box does not pin %.1f GB of host memory (gear_hip_host_alloc: %s)"
+                    % (nbytes / 1e9, lib.gear_hip_error_string(rc).decode()))
+    try:
+        g = torch.Generator(device="cuda")
+        g.manual_seed(5505)
+        piece_bytes = 1 << 30
+        announce("config 5 full size: filling the table from the device")
+        for o in range(0, nbytes, piece_bytes):
+            nb = min(piece_bytes, nbytes - o)
+            piece = torch.randint(0, 256, (nb,), dtype=torch.uint8, device="cuda", generator=g)
+            _cabi.call("gear_hip_memcpy", ctypes.c_void_p(host_ptr.value + o),
+                       ctypes.c_void_p(piece.data_ptr()), nb)
+        del piece
+        host = np.ctypeslib.as_array(ctypes.cast(host_ptr, ctypes.POINTER(ctypes.c_uint8)),
+                                     shape=(nbytes,))
+        rng = np.random.default_rng(5505)
+        pri = (rng.lognormal(0, 1, size=T * cap) ** 0.6).astype(np.float32)
+        u01 = rng.random(B, dtype=np.float32)
+        prefix = ops.prefix_sum(torch.from_numpy(pri).cuda())
+        flat, idxs, tss, lens = ops.sample_sorted(prefix, torch.from_numpy(u01).cuda(),
+                                                  unit_uniforms=True, trajectory_length=T)
+        dsts = [torch.full((B, SPAN * sb), 0xA5, dtype=torch.uint8, device="cuda")
+                for sb in STEP_BYTES]
+        cols = [dict(dst=dsts[c], ofst=OFST, span=SPAN, step_bytes=STEP_BYTES[c],
+                     col_base=int(accu[c]) * T, pad_head=True, zero_fill=True) for c in range(4)]
+        announce("config 5 full size: gather of 2048 windows x 4 columns from host memory")
+        ops.subcopy_multi(dev_ptr.value, idxs, tss, lens, S, cols)
+        torch.cuda.synchronize()
+        hi, ht = idxs.cpu().numpy(), tss.cpu().numpy()
+        assert np.array_equal(lens.cpu().numpy(), ht + 1)
+        assert hi.max() * S > 2 ** 35 and (ht < SPAN - 1).any() and hi.max() < cap
+        announce("config 5 full size: checking every window against the host bytes")
+        for c in range(4):
+            sb = STEP_BYTES[c]
+            got = dsts[c].cpu().numpy()
+            for w in range(B):
+                first = max(int(ht[w]) + 1 - SPAN, 0)
+                steps = int(ht[w]) + 1 - first
+                a = int(hi[w]) * S + int(accu[c]) * T + first * sb
+                assert np.array_equal(got[w, (SPAN - steps) * sb:], host[a:a + steps * sb]), (c, w)
+                assert not got[w, :(SPAN - steps) * sb].any(), (c, w)
     finally:
         torch.cuda.synchronize()
         assert lib.gear_hip_host_free(host_ptr) == 0

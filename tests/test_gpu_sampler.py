@@ -517,3 +517,57 @@ def test_chained_scans_on_two_streams_next_to_a_busy_gpu():
         for si in range(2):
             for j in range(len(pri)):
                 assert torch.equal(outs[si][j], ref[j])
+
+
+def test_select_with_lookups_equals_the_separate_calls(oracle):
+    """gear_hip_sample_lookup_f64 / gear_hip_sort_lookup_i64 / gear_hip_lookup_i64 against the
+    chain they fold (search -> sort -> indices[p] -> - offset -> timesteps[local]) on both sides
+    of the 4096-entry ranking sort, with an index offset, and against numpy."""
+    from gear_amd import ops
+    rng = np.random.default_rng(1234)
+    for n, num, offset in ((1, 1, 0), (5_000, 257, 0), (100_000, 4096, 1_000_000),
+                           (100_000, 4097, 77), (1_000_000, 20_000, 5)):
+        announce("select + look-ups n=%d num=%d offset=%d" % (n, num, offset))
+        pri = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+        if n > 10:
+            pri[rng.integers(0, n, size=n // 7)] = 0.0           # never drawn
+        pri[0] = max(pri[0], 0.5)
+        lengths = rng.integers(1, 1001, size=n).astype(np.int64)
+        indices = np.arange(n, dtype=np.int64) + offset          # ascending, as a loader's are
+        u = rng.random(num, dtype=np.float32)
+        dpri, dlen, dind, du = _dev(pri), _dev(lengths), _dev(indices), _dev(u)
+        prefix = ops.prefix_sum(dpri)
+        sampled, local, lens = ops.sample_lookup(prefix, du, index_table=dind, index_offset=offset,
+                                                 lengths_table=dlen)
+        pos = ops.sample_sorted(prefix, du, unit_uniforms=True)
+        torch.cuda.synchronize()
+        hpos = pos.cpu().numpy()
+        exp_pos = np.sort(oracle.upper_bound_f64(prefix.cpu().numpy(), u, unit_uniforms=True))
+        assert np.array_equal(hpos, exp_pos)
+        assert np.array_equal(sampled.cpu().numpy(), indices[exp_pos])
+        assert np.array_equal(local.cpu().numpy(), exp_pos)
+        assert np.array_equal(lens.cpu().numpy(), lengths[exp_pos])
+        # identity index table, only the lengths asked for
+        s2, l2, n2 = ops.sample_lookup(prefix, du, lengths_table=dlen)
+        torch.cuda.synchronize()
+        assert np.array_equal(s2.cpu().numpy(), exp_pos) and np.array_equal(n2.cpu().numpy(), lengths[exp_pos])
+        # uniform draws: positions given, with duplicates
+        draws = rng.integers(0, n, size=num).astype(np.int64)
+        s3, l3, n3 = ops.sort_lookup(_dev(draws), n, index_table=dind, index_offset=offset,
+                                     lengths_table=dlen)
+        torch.cuda.synchronize()
+        sd = np.sort(draws)
+        assert np.array_equal(s3.cpu().numpy(), indices[sd])
+        assert np.array_equal(l3.cpu().numpy(), sd) and np.array_equal(n3.cpu().numpy(), lengths[sd])
+        # positions in their own order (a top-k's selection), entries outside the tables read 0
+        order = draws.copy()
+        order[::97] = n + 3
+        s4, l4, n4 = ops.lookup(_dev(order), index_table=dind, index_offset=offset, lengths_table=dlen)
+        torch.cuda.synchronize()
+        inside = order < n
+        exp_s = np.where(inside, indices[np.minimum(order, n - 1)], 0)
+        exp_l = exp_s - offset
+        ok_l = (exp_l >= 0) & (exp_l < n)
+        exp_n = np.where(ok_l, lengths[np.clip(exp_l, 0, n - 1)], 0)
+        assert np.array_equal(s4.cpu().numpy(), exp_s) and np.array_equal(l4.cpu().numpy(), exp_l)
+        assert np.array_equal(n4.cpu().numpy(), exp_n)
