@@ -489,21 +489,35 @@ def run_config1(args):
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(args.steps)]
 
+    # the loader's step after the draws, in two calls: ascending sort of the drawn trajectories
+    # with the look-up of their recorded lengths (all 64 here) in the same launch, then the
+    # gather of all columns through a plan made once (same batch tensors every step)
+    lengths_table = torch.full((4096,), 64, dtype=torch.int64, device="cuda")
+    idx = torch.empty(B, dtype=torch.int64, device="cuda")
+    loc = torch.empty(B, dtype=torch.int64, device="cuda")
+    plan = ops.GatherPlan(table, tab.traj_stride, cols, B)
+
+    def select(d):
+        ops.sort_lookup(d, 4096, lengths_table=lengths_table, sampled_out=idx, local_out=loc,
+                        lens_out=lens)
+
     def step(i, slot):
-        idx = ops.sort_i64(draws[i], key_bits=12)
+        select(draws[i])
         if slot is not None:
             ev[slot][0].record()
-        ops.subcopy_multi(table, idx, tss, lens, tab.traj_stride, cols)
+        plan.run(idx, tss, lens)
         if slot is not None:
             ev[slot][1].record()
 
     ms = _time_steps(torch, step, args.steps, args.warmup)
     gms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
     cur = torch.empty(B, dtype=torch.int64, device="cuda")
-    ms_graph = _time_graph(
-        torch, lambda: ops.subcopy_multi(table, ops.sort_i64(cur, key_bits=12), tss, lens,
-                                         tab.traj_stride, cols),
-        lambda i: cur.copy_(draws[i]), args.steps, args.warmup)
+
+    def body():
+        select(cur)
+        plan.run(idx, tss, lens)
+
+    ms_graph = _time_graph(torch, body, lambda i: cur.copy_(draws[i]), args.steps, args.warmup)
     alg = 2 * B * tab.traj_stride
     host = table.cpu().numpy()
     hd = [np.zeros((B, 64 * sb), np.uint8) for sb in tab.step_bytes]
@@ -643,15 +657,27 @@ def run_config3(args):
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(args.steps)]
 
-    def step(i, slot):
+    # length-weighted draw, then sort + length look-up in one launch, the start offsets, and the
+    # gather through a plan made once (same batch tensors every step)
+    pos = torch.empty(B, dtype=torch.int64, device="cuda")
+    traj = torch.empty(B, dtype=torch.int64, device="cuda")
+    loc = torch.empty(B, dtype=torch.int64, device="cuda")
+    lens = torch.empty(B, dtype=torch.int64, device="cuda")
+    start = torch.empty(B, dtype=torch.int64, device="cuda")
+    plan = ops.GatherPlan(table, tab.traj_stride, cols, B)
+
+    def select(ua, ub):
         ops.prefix_sum_i64(lengths, out=prefix)
-        traj = ops.upper_bound_i64(prefix, u1[i], unit_uniforms=True)
-        traj = ops.sort_i64(traj, key_bits=17)
-        lens = ops.take_i64(lengths, traj)
-        start = (u2[i] * (lens - (span - 1)).double()).long()   # synthetic start offsets (input)
+        ops.upper_bound_i64(prefix, ua, unit_uniforms=True, idx_out=pos)
+        ops.sort_lookup(pos, tab.capacity, lengths_table=lengths, sampled_out=traj, local_out=loc,
+                        lens_out=lens)
+        start.copy_(ub * (lens - (span - 1)))   # synthetic start offsets (an input of the config)
+
+    def step(i, slot):
+        select(u1[i], u2[i])
         if slot is not None:
             ev[slot][0].record()
-        ops.subcopy_multi(table, traj, start, lens, tab.traj_stride, cols)
+        plan.run(traj, start, lens)
         if slot is not None:
             ev[slot][1].record()
 
@@ -660,11 +686,8 @@ def run_config3(args):
     uc = torch.empty((2, B), dtype=torch.float64, device="cuda")
 
     def body():
-        ops.prefix_sum_i64(lengths, out=prefix)
-        traj = ops.sort_i64(ops.upper_bound_i64(prefix, uc[0], unit_uniforms=True), key_bits=17)
-        lens = ops.take_i64(lengths, traj)
-        start = (uc[1] * (lens - (span - 1)).double()).long()
-        ops.subcopy_multi(table, traj, start, lens, tab.traj_stride, cols)
+        select(uc[0], uc[1])
+        plan.run(traj, start, lens)
 
     def feed(i):
         uc[0].copy_(u1[i])

@@ -79,6 +79,31 @@ def build_libgear_ext():
     return out
 
 
+SANITIZE_FLAGS = ["-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+                  "-fno-omit-frame-pointer", "-O1", "-g"]
+
+
+def build_sanitized(outdir):
+    """The host C++ layer (pybind module) and the CPU oracle compiled with AddressSanitizer and
+    UndefinedBehaviorSanitizer into `outdir`: host code only, for tests/host_sanitizers.py.  The
+    HIP library is linked as it is (never a sanitized GPU build).  Returns the two paths."""
+    import pybind11
+    os.makedirs(outdir, exist_ok=True)
+    host = os.path.join(CSRC, "host")
+    srcs = sorted(os.path.join(host, f) for f in os.listdir(host) if f.endswith(".cc"))
+    suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+    module = os.path.join(outdir, "_libgear" + suffix)
+    _run(["g++", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"] + SANITIZE_FLAGS +
+         ["-I", INCLUDE, "-I", host, "-I", pybind11.get_include(),
+          "-I", sysconfig.get_paths()["include"]] + srcs +
+         ["-o", module, "-L", _PKG, "-lgearhip", "-Wl,-rpath," + _PKG, "-ldl", "-lpthread"])
+    oracle = os.path.join(outdir, "liboracle.so")
+    _run(["gcc", "-std=c11", "-fPIC", "-shared", "-fvisibility=hidden", "-fopenmp", "-Wall",
+          "-Wextra"] + SANITIZE_FLAGS +
+         [os.path.join(_ROOT, "oracle", "gear_oracle.c"), "-o", oracle, "-lm"])
+    return module, oracle
+
+
 def build_all(verbose=False):
     build_libgearhip(verbose)
     if os.path.isdir(os.path.join(CSRC, "host")):

@@ -9,7 +9,18 @@ import os as _os
 import sys as _sys
 
 try:
-    from . import _libgear
+    _alt = _os.environ.get("GEAR_LIBGEAR_MODULE")
+    if _alt:
+        # another build of the same module (the host-sanitizer run of tests/host_sanitizers.py)
+        import importlib.machinery as _mach
+        import importlib.util as _util
+        _loader = _mach.ExtensionFileLoader(__name__ + "._libgear", _alt)
+        _spec = _util.spec_from_file_location(__name__ + "._libgear", _alt, loader=_loader)
+        _libgear = _util.module_from_spec(_spec)
+        _loader.exec_module(_libgear)
+        _sys.modules[__name__ + "._libgear"] = _libgear
+    else:
+        from . import _libgear
 except ImportError as _e:  # pragma: no cover - only without a build
     raise ImportError(
         "gear_amd.libgear: the native module is not built; run "

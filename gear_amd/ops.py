@@ -5,6 +5,7 @@ stream.  All arithmetic happens in libgearhip.so; nothing in this module compute
 nothing falls back to torch or to the CPU.
 """
 import ctypes
+import functools
 
 import torch
 
@@ -27,13 +28,15 @@ def _stream_value(device=None):
 
 
 def _stream():
-    return ctypes.c_void_p(_stream_value())
+    # (plain integers: ctypes converts them for the void* parameters itself, and building a
+    # c_void_p object per argument is a measurable part of a small step)
+    return _stream_value()
 
 
 def _ptr(t):
     if t is None:
         return None
-    return ctypes.c_void_p(t.data_ptr())
+    return t.data_ptr()
 
 
 def _need(t, dtype, name, device=True):
@@ -51,12 +54,18 @@ def _need(t, dtype, name, device=True):
 def _src_ptr(src):
     """Table base: an int address (MemoryPtr-style), or a tensor (device, or pinned host)."""
     if isinstance(src, int):
-        return ctypes.c_void_p(src)
+        return src
     if isinstance(src, torch.Tensor):
-        return ctypes.c_void_p(src.data_ptr())
+        return src.data_ptr()
     if hasattr(src, "address"):
-        return ctypes.c_void_p(int(src.address))
+        return int(src.address)
     raise TypeError("unsupported table source %r" % type(src))
+
+
+@functools.lru_cache(maxsize=512)
+def _ws_bytes(query, *sizes):
+    """Result of a *_workspace_bytes query of the library (a pure function of the sizes)."""
+    return getattr(load(), query)(*[int(v) for v in sizes])
 
 
 class _Workspace:
@@ -259,7 +268,7 @@ def prefix_sum(priorities, out=None):
         _need(out, torch.float64, "out")
         if out.numel() < n:
             raise ValueError("out is too small")
-    nbytes = load().gear_hip_scan_workspace_bytes(n)
+    nbytes = _ws_bytes("gear_hip_scan_workspace_bytes", n)
     ws = _ws.get("scan", nbytes, priorities.device)
     call("gear_hip_scan_f32_f64", _ptr(priorities), _ptr(out), n, _ptr(ws), ws.numel(), _stream())
     return out
@@ -297,7 +306,7 @@ class PrefixState:
         n = priorities.numel()
         if self.out is None or self._n != n or self.out.device != priorities.device:
             self.out = torch.empty(n, dtype=torch.float64, device=priorities.device)
-            nbytes = load().gear_hip_scan_workspace_bytes(n)
+            nbytes = _ws_bytes("gear_hip_scan_workspace_bytes", n)
             self._ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8,
                                    device=priorities.device)
             self._n = n
@@ -322,7 +331,7 @@ def prefix_sum_i64(weights, out=None):
         out = torch.empty(n, dtype=torch.int64, device=weights.device)
     else:
         _need(out, torch.int64, "out")
-    nbytes = load().gear_hip_scan_workspace_bytes(n)
+    nbytes = _ws_bytes("gear_hip_scan_workspace_bytes", n)
     ws = _ws.get("scan", nbytes, weights.device)
     call("gear_hip_scan_i64", _ptr(weights), _ptr(out), n, _ptr(ws), ws.numel(), _stream())
     return out
@@ -333,7 +342,7 @@ def sum_f32(values, out=None, out_f64=None):
     n = values.numel()
     if out is None:
         out = torch.empty(1, dtype=torch.float32, device=values.device)
-    nbytes = load().gear_hip_sum_workspace_bytes(n)
+    nbytes = _ws_bytes("gear_hip_sum_workspace_bytes", n)
     ws = _ws.get("sum", nbytes, values.device)
     call("gear_hip_sum_f32", _ptr(values), n, _ptr(out), _ptr(out_f64), _ptr(ws), ws.numel(),
          _stream())
@@ -357,7 +366,7 @@ def upper_bound(prefix, u, *, unit_uniforms=False, idx_out=None, priorities=None
             raise ValueError("priorities and prefix differ in length")
         if weights_out is None:
             weights_out = torch.empty(num, dtype=torch.float32, device=u.device)
-        nbytes = load().gear_hip_search_workspace_bytes(num)
+        nbytes = _ws_bytes("gear_hip_search_workspace_bytes", num)
         ws = _ws.get("search", nbytes, u.device)
     call("gear_hip_upper_bound_f64", _ptr(prefix), prefix.numel(), _ptr(u), num,
          int(bool(unit_uniforms)), _ptr(idx_out), _ptr(priorities), float(beta),
@@ -381,7 +390,7 @@ def sample_sorted(prefix, u, *, unit_uniforms=True, sorted_out=None, trajectory_
         idxs = idxs if idxs is not None else torch.empty(num, dtype=torch.int64, device=dev)
         tss = tss if tss is not None else torch.empty(num, dtype=torch.int64, device=dev)
         lens = lens if lens is not None else torch.empty(num, dtype=torch.int64, device=dev)
-    nbytes = load().gear_hip_sample_workspace_bytes(num)
+    nbytes = _ws_bytes("gear_hip_sample_workspace_bytes", num)
     ws = _ws.get("sample", nbytes, dev)
     call("gear_hip_sample_sorted_f64", _ptr(prefix), prefix.numel(), _ptr(u), num,
          int(bool(unit_uniforms)), _ptr(sorted_out), int(trajectory_length), int(modulo),
@@ -414,7 +423,7 @@ def sample_lookup(prefix, u, *, unit_uniforms=True, index_table=None, index_offs
     if lengths_table is not None:
         _need(lengths_table, torch.int64, "lengths_table")
     sampled, local, lens = _lookup_outputs(num, dev, lengths_table, sampled_out, local_out, lens_out)
-    ws = _ws.get("sample", load().gear_hip_sample_workspace_bytes(num), dev)
+    ws = _ws.get("sample", _ws_bytes("gear_hip_sample_workspace_bytes", num), dev)
     call("gear_hip_sample_lookup_f64", _ptr(prefix), prefix.numel(), _ptr(u), num,
          int(bool(unit_uniforms)), _ptr(index_table), int(index_offset), _ptr(lengths_table),
          lengths_table.numel() if lengths_table is not None else 0, _ptr(sampled), _ptr(local),
@@ -433,7 +442,7 @@ def sort_lookup(positions, bound, *, index_table=None, index_offset=0, lengths_t
     if lengths_table is not None:
         _need(lengths_table, torch.int64, "lengths_table")
     sampled, local, lens = _lookup_outputs(num, dev, lengths_table, sampled_out, local_out, lens_out)
-    ws = _ws.get("sample", load().gear_hip_sample_workspace_bytes(num), dev)
+    ws = _ws.get("sample", _ws_bytes("gear_hip_sample_workspace_bytes", num), dev)
     call("gear_hip_sort_lookup_i64", _ptr(positions), num, int(bound), _ptr(index_table),
          index_table.numel() if index_table is not None else 0, int(index_offset),
          _ptr(lengths_table), lengths_table.numel() if lengths_table is not None else 0,
@@ -478,7 +487,7 @@ def sort_i64(keys, vals=None, key_bits=63):
     if vals is not None:
         _need(vals, torch.int64, "vals")
         vals_out = torch.empty_like(vals)
-    nbytes = load().gear_hip_sort_workspace_bytes(num)
+    nbytes = _ws_bytes("gear_hip_sort_workspace_bytes", num)
     ws = _ws.get("sort", nbytes, keys.device)
     call("gear_hip_sort_i64", _ptr(keys), _ptr(keys_out), _ptr(vals), _ptr(vals_out), num,
          int(key_bits), _ptr(ws), ws.numel(), _stream())
@@ -493,7 +502,7 @@ def topk(priorities, k, *, sorted_by_value=True, want_values=True, warm=False, w
     n = priorities.numel()
     idx = torch.empty(k, dtype=torch.int64, device=priorities.device)
     vals = torch.empty(k, dtype=torch.float32, device=priorities.device) if want_values else None
-    nbytes = load().gear_hip_topk_workspace_bytes(n, k)
+    nbytes = _ws_bytes("gear_hip_topk_workspace_bytes", n, k)
     ws = workspace if workspace is not None else _ws.get("topk", nbytes, priorities.device)
     if ws.numel() < nbytes:
         raise ValueError("top-k workspace holds %d bytes, %d needed" % (ws.numel(), nbytes))
@@ -514,7 +523,7 @@ class TopKState:
     def select(self, priorities, k, *, sorted_by_value=True, want_values=True):
         n = priorities.numel()
         shape = (n, int(k), bool(sorted_by_value), priorities.device)
-        nbytes = load().gear_hip_topk_workspace_bytes(n, k)
+        nbytes = _ws_bytes("gear_hip_topk_workspace_bytes", n, k)
         warm = self._shape == shape
         if self._ws is None or self._ws.numel() < nbytes or self._ws.device != priorities.device:
             self._ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8,
@@ -537,7 +546,7 @@ def scatter(weights, idx, values, *, unique_indices=False):
         raise ValueError("idx and values differ in length")
     ws = None
     if not unique_indices:
-        nbytes = load().gear_hip_scatter_workspace_bytes(num)
+        nbytes = _ws_bytes("gear_hip_scatter_workspace_bytes", num)
         ws = _ws.get("scatter", nbytes, weights.device)
     fn = "gear_hip_scatter_f32" if weights.dtype == torch.float32 else "gear_hip_scatter_i64"
     call(fn, _ptr(weights), weights.numel(), _ptr(idx), _ptr(values), num,

@@ -8,6 +8,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+def pytest_addoption(parser):
+    parser.addoption("--host-sanitizers", action="store_true", default=False,
+                     help="also run tests/host_sanitizers.py (ASan + UBSan builds of the host C++ "
+                          "layer and the oracle under the CPU tests; about two minutes)")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run on the GPU box)")
 

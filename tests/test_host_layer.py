@@ -351,3 +351,16 @@ def test_loader_partition_and_rank_order_on_one_rank():
     topk_loader = OfflineLoader(ds, 3, ModelParallelismUnit(device="cpu"), "Topk",
                                 [{"name": "obs", "offset": 0, "length": 4}])
     assert isinstance(topk_loader._sampler, gear.sampler.TopKSampler)
+
+
+def test_host_code_is_clean_under_address_and_ub_sanitizers(request):
+    """The host C++ layer and the oracle rebuilt with -fsanitize=address,undefined and run under
+    the CPU tests of this directory (tests/host_sanitizers.py); opt-in: pytest --host-sanitizers."""
+    if not request.config.getoption("--host-sanitizers"):
+        pytest.skip("run with --host-sanitizers (rebuilds the host code with ASan + UBSan)")
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "tests", "host_sanitizers.py")],
+                       cwd=root, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout[-4000:]
