@@ -687,7 +687,11 @@ __global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
   __shared__ __align__(16) uint32_t h[kHintedBins];  // the bins from the hint upwards
   __shared__ uint64_t queue[kWavesPerBlock][kQueueCap];
   __shared__ uint32_t s_touched[kHintedBins / kWave];  // runs of 64 bins that hold a count
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // (the same in every lane of a wave: said so, everything that follows from it -- the wave's
+  // range, the number of its steps -- stays in scalar registers and branches on it are taken by
+  // whole waves, without copies of the loaded values where the paths meet)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   const int64_t begin = gw * wave_len;
   const int64_t end = begin + wave_len < n ? begin + wave_len : n;
@@ -697,16 +701,18 @@ __global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
   // Loads of whole steps carry no test and no branch (a branch around a load makes the compiler
   // wait for every load where the paths meet); a step beyond the last whole one is loaded from
   // the last one's place and not looked at.
+  // (a wave without a whole step loads the first steps of the input, which exist, and does not
+  // look at them: the first loads then need no branch either)
+  const float *lbase = whole > 0 ? base : p;
+  const int last = whole > 0 ? whole - 1 : 0;
   auto load_step = [&](int step, f4 &v) {
-    const int st = step < whole ? step : whole - 1;
-    v = *reinterpret_cast<const f4 *>(base + (int64_t)st * kStep + lane * 4);
+    const int st = step < last ? step : last;
+    v = *reinterpret_cast<const f4 *>(lbase + (int64_t)st * kStep + lane * 4);
   };
   // the first loads go out before the histogram is cleared
   f4 qa[kAhead], qb[kAhead];
-  if (whole > 0) {
 #pragma unroll
-    for (int a = 0; a < kAhead; ++a) load_step(a, qa[a]);
-  }
+  for (int a = 0; a < kAhead; ++a) load_step(a, qa[a]);
   static_assert(kHintedBins == kThreads * 4, "one 16-byte store per thread clears the histogram");
   *reinterpret_cast<u32x4 *>(&h[tid * 4]) = u32x4{0u, 0u, 0u, 0u};
   if (tid < kHintedBins / kWave) s_touched[tid] = 0u;
@@ -742,20 +748,42 @@ __global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
     }
     queued = (uint32_t)__builtin_amdgcn_readfirstlane((int)(queued + total));
   };
-  for (int st = 0; st < whole && !given_up;) {
+  // Two groups of kAhead steps take turns: while one is looked at, the loads of the other are
+  // under way.  Inside the loop the next group lies wholly inside the range, so its loads carry
+  // no test (a branch around a load makes the compiler copy the loaded registers where the
+  // paths meet, and wait for the load there); the last one or two groups are handled after it,
+  // with loads past the range redirected to the last step and not looked at.
+  int st = 0;  // qa holds the steps st .. st + kAhead - 1
+  while (!given_up && st + 2 * kAhead <= whole) {
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+      qb[a] = *reinterpret_cast<const f4 *>(lbase + (int64_t)(st + kAhead + a) * kStep + lane * 4);
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+      if (!given_up) take((st + a) * kStep, qa[a]);
+    st += kAhead;
+    if (given_up || st + 2 * kAhead > whole) {
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) qa[a] = qb[a];
+      break;
+    }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+      qa[a] = *reinterpret_cast<const f4 *>(lbase + (int64_t)(st + kAhead + a) * kStep + lane * 4);
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a)
+      if (!given_up) take((st + a) * kStep, qb[a]);
+    st += kAhead;
+  }
+  if (!given_up && st < whole) {
 #pragma unroll
     for (int a = 0; a < kAhead; ++a) load_step(st + kAhead + a, qb[a]);
 #pragma unroll
     for (int a = 0; a < kAhead; ++a)
       if (st + a < whole && !given_up) take((st + a) * kStep, qa[a]);
-    st += kAhead;
-    if (st >= whole || given_up) break;
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a) load_step(st + kAhead + a, qa[a]);
 #pragma unroll
     for (int a = 0; a < kAhead; ++a)
-      if (st + a < whole && !given_up) take((st + a) * kStep, qb[a]);
-    st += kAhead;
+      if (st + kAhead + a < whole && !given_up) take((st + kAhead + a) * kStep, qb[a]);
   }
   if (!given_up && whole * kStep < len) {
     // the ragged end of the input, in the one wave that holds it; what lies beyond reads as
@@ -1334,10 +1362,16 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
   auto emit = [&](bool selected, bool is_eq, uint32_t pos, uint32_t e, uint32_t index, uint32_t key,
                   auto have, float value) {
     selected = selected && pos < (uint32_t)k;  // out of step only with NaN priorities
+    // (a listed entry's priority follows from its key, except for the two zeros, which share
+    // one: only those are read from the input -- a gather of every selected value costs 8 MB of
+    // cache lines for 65536 entries)
+    auto value_of = [&]() {
+      return decltype(have)::value ? value : (key != 0x80000000u ? key_to_float(key) : p[index]);
+    };
     if (FLAVOUR == kDirect) {
       if (selected) {
         indices_out[pos] = (int64_t)index;
-        if (values_out) values_out[pos] = decltype(have)::value ? value : p[index];
+        if (values_out) values_out[pos] = value_of();
       }
     } else if (FLAVOUR == kPairs) {
       if (selected) {
@@ -1349,7 +1383,7 @@ __global__ __launch_bounds__(kThreads) void write_kernel(
       // bucket sort skips them (it takes keys above T only)
       if (selected && is_eq && ties_at + e < (uint32_t)k) {
         indices_out[ties_at + e] = (int64_t)index;
-        if (values_out) values_out[ties_at + e] = decltype(have)::value ? value : p[index];
+        if (values_out) values_out[ties_at + e] = value_of();
       }
       if (selected) {
         ckey[pos] = key;
