@@ -23,7 +23,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per gather launch on config 4, from the two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE, each scaled by a 1 GiB plain copy in the same run) summarised in
 # profiles/subcopy_multi_kernel_config4_hbm_traffic.txt
-MEASURED_GATHER_TRAFFIC_BYTES = 3486581717
+MEASURED_GATHER_TRAFFIC_BYTES = 3486579262
 
 
 def log(msg):
