@@ -571,3 +571,29 @@ def test_select_with_lookups_equals_the_separate_calls(oracle):
         exp_n = np.where(ok_l, lengths[np.clip(exp_l, 0, n - 1)], 0)
         assert np.array_equal(s4.cpu().numpy(), exp_s) and np.array_equal(l4.cpu().numpy(), exp_l)
         assert np.array_equal(n4.cpu().numpy(), exp_n)
+
+
+def test_staggered_start_of_the_chained_scan_changes_no_bit():
+    """GEAR_HIP_SCAN_STAGGER_PS (read at every call): workgroups of the chained kernel's first
+    wave start a little after one another above 512 ranges.  Off, at the default and four times
+    as long, the prefix has the same bits."""
+    from gear_amd import ops
+    rng = np.random.default_rng(4321)
+    pri = _dev((rng.lognormal(0, 1, size=10_000_003) ** 0.6).astype(np.float32))
+    old = os.environ.get("GEAR_HIP_SCAN_STAGGER_PS")
+    try:
+        outs = []
+        for ps in ("0", None, "20000"):
+            if ps is None:
+                os.environ.pop("GEAR_HIP_SCAN_STAGGER_PS", None)
+            else:
+                os.environ["GEAR_HIP_SCAN_STAGGER_PS"] = ps
+            announce("chained scan, stagger %s ps" % ps)
+            outs.append(ops.prefix_sum(pri).clone())
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+    finally:
+        if old is None:
+            os.environ.pop("GEAR_HIP_SCAN_STAGGER_PS", None)
+        else:
+            os.environ["GEAR_HIP_SCAN_STAGGER_PS"] = old
