@@ -675,6 +675,14 @@ constexpr int kQueueCap = 512;  // candidates per wave held in LDS; longer lists
 // histogram in memory (a sweep over all 16384 bins by every workgroup cost 4 us of a 16 us
 // launch).  A wave whose candidates outgrow the queue gives its list up (the later launches read
 // its range again) and counts the candidates of its range straight into the histogram.
+// Where a candidate's bin is counted: from the hint's bin upwards.  (A map laid out around NaN
+// samples -- NaN is not a valid priority -- can take an infinity for a candidate whose bin lies
+// below the hint's: whatever the result then is, the count stays inside the histogram.)
+__device__ __forceinline__ uint32_t counted_bin(uint32_t bin, uint32_t bin_base) {
+  const uint32_t at = bin >= bin_base ? bin - bin_base : 0u;
+  return at < (uint32_t)kHintedBins ? at : (uint32_t)kHintedBins - 1u;
+}
+
 __device__ __forceinline__ uint32_t lanes_before(uint64_t mask, uint32_t acc) {
   return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
                                    __builtin_amdgcn_mbcnt_lo((uint32_t)mask, acc));
@@ -807,7 +815,7 @@ __global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
       for (int j = 0; j < 4; ++j) {
         const bool cand = e0 + j < end && q[j] >= lo_f;
         if (wave_ballot(cand) == 0ull) continue;
-        const uint32_t bin = bin_of(map, order_key(q[j])) - bin_base;
+        const uint32_t bin = counted_bin(bin_of(map, order_key(q[j])), bin_base);
         count_add(h, bin, cand);
         if (cand) s_touched[bin / kWave] = 1u;
       }
@@ -818,7 +826,7 @@ __global__ __launch_bounds__(kThreads) void level0_hinted_kernel(
   for (uint32_t i = (uint32_t)lane; i < queued; i += kWave) {
     const uint64_t ent = wq[i];
     const uint32_t key = order_key(__uint_as_float((uint32_t)(ent >> 32)));
-    const uint32_t bin = bin_of(map, key) - bin_base;
+    const uint32_t bin = counted_bin(bin_of(map, key), bin_base);
     atomicAdd(&h[bin], 1u);
     s_touched[bin / kWave] = 1u;
     list[i] = ((uint64_t)key << 32) | (uint32_t)ent;

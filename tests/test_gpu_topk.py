@@ -109,7 +109,14 @@ def test_topk_nan_priorities_stay_inside_the_outputs():
     n = 300_000
     for frac, k in ((0.001, 4_096), (0.5, 4_096), (1.0, 4_096), (0.5, 20_000), (1.0, 20_000)):
         w = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
-        w[rng.random(n) < frac] = np.nan
+        nan = rng.random(n) < frac
+        w[nan] = np.nan
+        # NaNs of either sign next to infinities: a bin map laid out around NaN samples may take
+        # the infinities for candidates whose bins lie below the bound's
+        bits = w.view(np.uint32)
+        bits[nan & (rng.random(n) < 0.5)] |= np.uint32(0x80000000)
+        w[rng.permutation(n)[:2_000]] = np.inf
+        w[rng.permutation(n)[:1_000]] = -np.inf
         dw = _dev(w)
         for by_value in (0, 1):
             vals = torch.full((k + 1024,), -7.0, dtype=torch.float32, device="cuda")
