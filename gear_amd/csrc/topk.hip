@@ -439,29 +439,46 @@ __device__ __forceinline__ void load_quad(const float *__restrict__ p, int64_t e
 // the previous kAhead are handed to f(e0, q) -- e0 the index of the lane's first element, q its
 // four values; elements at or beyond `end` hold 0 and must be skipped (e0 + j < end).  Every
 // lane of the wave calls f the same number of times, so f may ballot.
+// The loads of the steps that lie inside the range carry no test and no branch: the compiler
+// waits for every load that a branch goes around where the paths meet, one round trip to memory
+// per step instead of one per kAhead steps.  A step beyond the last whole one is loaded from the
+// last one's place and not looked at; what is left of the range after its whole steps (the end
+// of the input: the last wave) is loaded element by element, once.
+__device__ const float g_zero_step[kStep] = {};  // something to load where a range has no whole step
+__device__ __forceinline__ f4 load_whole_step(const float *lane_base, int step, int last) {
+  const int st = step < last ? step : last;
+  return *reinterpret_cast<const f4 *>(lane_base + (int64_t)st * kStep);
+}
 template <typename F>
 __device__ __forceinline__ void stream_range(const float *__restrict__ p, int64_t begin,
                                              int64_t end, int lane, F f) {
   if (begin >= end) return;
-  float q[kAhead][4];
+  const int whole = (int)((end - begin) / kStep);
+  if (whole > 0) {
+    const float *lane_base = p + begin + lane * 4;
+    f4 q[kAhead];
 #pragma unroll
-  for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
-  for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
-    float qn[kAhead][4];
-    const int64_t s1 = s0 + kAhead * kStep;
-    if (s1 < end) {
+    for (int a = 0; a < kAhead; ++a) q[a] = load_whole_step(lane_base, a, whole - 1);
+    for (int s = 0; s < whole; s += kAhead) {
+      f4 qn[kAhead];
 #pragma unroll
-      for (int a = 0; a < kAhead; ++a) load_quad(p, s1 + (int64_t)a * kStep + lane * 4, end, qn[a]);
+      for (int a = 0; a < kAhead; ++a) qn[a] = load_whole_step(lane_base, s + kAhead + a, whole - 1);
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) {
+        if (s + a < whole) {
+          const float v[4] = {q[a][0], q[a][1], q[a][2], q[a][3]};
+          f(begin + (int64_t)(s + a) * kStep + lane * 4, v);
+        }
+      }
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) q[a] = qn[a];
     }
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a) {
-      const int64_t e0 = s0 + (int64_t)a * kStep + lane * 4;
-      if (s0 + (int64_t)a * kStep < end) f(e0, q[a]);
-    }
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) q[a][j] = qn[a][j];
+  }
+  const int64_t t0 = begin + (int64_t)whole * kStep;
+  if (t0 < end) {
+    float v[4];
+    load_quad(p, t0 + lane * 4, end, v);
+    f(t0 + lane * 4, v);
   }
 }
 
@@ -470,35 +487,40 @@ __device__ __forceinline__ void stream_range(const float *__restrict__ p, int64_
 // The caller asks for the first kAhead steps itself (stream_first), ahead of work that does
 // not depend on them.
 __device__ __forceinline__ void stream_first(const float *__restrict__ p, int64_t begin, int64_t end,
-                                             int lane, float (&q)[kAhead][4]) {
+                                             int lane, f4 (&q)[kAhead]) {
+  // (a wave without a whole step loads zeros that it does not look at: no branch here either)
+  const int whole = begin < end ? (int)((end - begin) / kStep) : 0;
+  const float *lane_base = (whole > 0 ? p + begin : g_zero_step) + lane * 4;
 #pragma unroll
-  for (int a = 0; a < kAhead; ++a) load_quad(p, begin + (int64_t)a * kStep + lane * 4, end, q[a]);
+  for (int a = 0; a < kAhead; ++a) q[a] = load_whole_step(lane_base, a, whole > 0 ? whole - 1 : 0);
 }
 template <typename F>
 __device__ __forceinline__ void stream_range_tagged(const float *__restrict__ p, int64_t begin,
-                                                    int64_t end, int lane, float (&q)[kAhead][4],
-                                                    F f) {
+                                                    int64_t end, int lane, f4 (&q)[kAhead], F f) {
   if (begin >= end) return;
-  for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
-    float qn[kAhead][4];
-    const int64_t s1 = s0 + kAhead * kStep;
-    if (s1 < end) {
+  const int whole = (int)((end - begin) / kStep);
+  if (whole > 0) {
+    const float *lane_base = p + begin + lane * 4;
+    for (int s = 0; s < whole; s += kAhead) {
+      f4 qn[kAhead];
 #pragma unroll
-      for (int a = 0; a < kAhead; ++a) load_quad(p, s1 + (int64_t)a * kStep + lane * 4, end, qn[a]);
+      for (int a = 0; a < kAhead; ++a) qn[a] = load_whole_step(lane_base, s + kAhead + a, whole - 1);
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) {
+        if (s + a < whole) {
+          const float v[4] = {q[a][0], q[a][1], q[a][2], q[a][3]};
+          f(begin + (int64_t)(s + a) * kStep + lane * 4, v, std::true_type{});
+        }
+      }
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a) q[a] = qn[a];
     }
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a) {
-      const int64_t w0 = s0 + (int64_t)a * kStep;
-      const int64_t e0 = w0 + lane * 4;
-      if (w0 + kStep <= end)
-        f(e0, q[a], std::true_type{});
-      else if (w0 < end)
-        f(e0, q[a], std::false_type{});
-    }
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) q[a][j] = qn[a][j];
+  }
+  const int64_t t0 = begin + (int64_t)whole * kStep;
+  if (t0 < end) {
+    float v[4];
+    load_quad(p, t0 + lane * 4, end, v);
+    f(t0 + lane * 4, v, std::false_type{});
   }
 }
 
@@ -509,35 +531,39 @@ template <typename F>
 __device__ __forceinline__ void stream_rows(const float *__restrict__ p, int64_t begin, int64_t end,
                                             int lane, F f) {
   if (begin >= end) return;
-  auto load_step = [&](int64_t s0, float (&q)[4]) {
+  const int whole = (int)((end - begin) / kStep);  // steps of four whole rows
+  if (whole > 0) {
+    const float *lane_base = p + begin + lane;
+    auto load_step = [&](int step, float (&q)[4]) {
+      const int st = step < whole - 1 ? step : whole - 1;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int64_t i = s0 + j * kWave + lane;
-      q[j] = i < end ? p[i] : 0.0f;
-    }
-  };
-  float q[kAhead][4];
+      for (int j = 0; j < 4; ++j) q[j] = lane_base[(int64_t)st * kStep + j * kWave];
+    };
+    float q[kAhead][4];
 #pragma unroll
-  for (int a = 0; a < kAhead; ++a) load_step(begin + (int64_t)a * kStep, q[a]);
-  for (int64_t s0 = begin; s0 < end; s0 += kAhead * kStep) {
-    float qn[kAhead][4];
-    const int64_t s1 = s0 + kAhead * kStep;
-    if (s1 < end) {
+    for (int a = 0; a < kAhead; ++a) load_step(a, q[a]);
+    for (int s = 0; s < whole; s += kAhead) {
+      float qn[kAhead][4];
 #pragma unroll
-      for (int a = 0; a < kAhead; ++a) load_step(s1 + (int64_t)a * kStep, qn[a]);
-    }
+      for (int a = 0; a < kAhead; ++a) load_step(s + kAhead + a, qn[a]);
 #pragma unroll
-    for (int a = 0; a < kAhead; ++a) {
+      for (int a = 0; a < kAhead; ++a) {
+        if (s + a < whole) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int64_t r0 = s0 + (int64_t)a * kStep + j * kWave;
-        if (r0 < end) f(r0 + lane, q[a][j], r0 + lane < end);
+          for (int j = 0; j < 4; ++j)
+            f(begin + (int64_t)(s + a) * kStep + j * kWave + lane, q[a][j], true);
+        }
       }
+#pragma unroll
+      for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) q[a][j] = qn[a][j];
     }
-#pragma unroll
-    for (int a = 0; a < kAhead; ++a)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) q[a][j] = qn[a][j];
+  }
+  // what is left after the whole steps: up to four rows, the last one ragged
+  for (int64_t r0 = begin + (int64_t)whole * kStep; r0 < end; r0 += kWave) {
+    const int64_t i = r0 + lane;
+    f(i, i < end ? p[i] : 0.0f, i < end);
   }
 }
 
@@ -867,7 +893,7 @@ __global__ __launch_bounds__(kThreads) void level0_kernel(const float *__restric
   const int64_t gw = (int64_t)blockIdx.x * kWavesPerBlock + wave;
   const int64_t begin = gw * wave_len;
   const int64_t end = begin + wave_len < n ? begin + wave_len : n;
-  float q0[kAhead][4];
+  f4 q0[kAhead];
   stream_first(p, begin, end, lane, q0);
   for (int i = tid; i < kBins0; i += kThreads) h[i] = 0u;
   const bool whole_ranges = state->hint_bin != kNoLists;
@@ -1553,17 +1579,11 @@ __device__ __forceinline__ void count_add(uint32_t *cnt, uint32_t d, bool valid)
 // LDS counter, one after the other.  Returns how many low bits of src[off, off+len) can still
 // differ (at most rem): the position of the highest bit in which two entries differ, plus one.
 // Called by every thread of the workgroup.
-__device__ __forceinline__ int differing_bits(const uint64_t *src, uint32_t off, uint32_t len,
-                                              int rem, SortShared &sh) {
+// (the second half of it: o and a are the OR and the AND of the entries this thread looked at)
+__device__ __forceinline__ int differing_bits_of(uint64_t o, uint64_t a, int rem, SortShared &sh) {
   const int tid = threadIdx.x;
   if (tid < 4) sh.bits_or_and[tid] = tid < 2 ? 0u : 0xffffffffu;
   __syncthreads();
-  uint64_t o = 0ull, a = ~0ull;
-  for (uint32_t i = tid; i < len; i += kSortThreads) {
-    const uint64_t x = src[off + i];
-    o |= x;
-    a &= x;
-  }
   for (int d = 32; d >= 1; d >>= 1) {  // the wave's lanes, then one atomic per wave and word
     o |= (uint64_t)__shfl_xor((unsigned long long)o, d, kWave);
     a &= (uint64_t)__shfl_xor((unsigned long long)a, d, kWave);
@@ -1580,6 +1600,26 @@ __device__ __forceinline__ int differing_bits(const uint64_t *src, uint32_t off,
   __syncthreads();
   if (rem < 64) diff &= (1ull << rem) - 1ull;
   return diff ? 64 - __builtin_clzll(diff) : 0;
+}
+__device__ __forceinline__ int differing_bits(const uint64_t *src, uint32_t off, uint32_t len,
+                                              int rem, SortShared &sh) {
+  uint64_t o = 0ull, a = ~0ull;
+  // (several loads under way per thread: out of global memory one at a time is a round trip each)
+  constexpr int kLoadsAhead = 8;
+  for (uint32_t i0 = threadIdx.x; i0 < len; i0 += kSortThreads * kLoadsAhead) {
+    uint64_t x[kLoadsAhead];
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u) {
+      const uint32_t i = i0 + (uint32_t)u * kSortThreads;
+      x[u] = src[off + (i < len ? i : 0u)];  // (beyond the end: the first entry once more)
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u) {
+      o |= x[u];
+      a &= x[u];
+    }
+  }
+  return differing_bits_of(o, a, rem, sh);
 }
 
 // Sorts the m entries a[0, m) (descending; only their low `bits` bits can differ) with b as the
@@ -1693,6 +1733,7 @@ struct BigShared {
   uint32_t gstart[kBigBins + 1];
   uint32_t off[kBigStack], len[kBigStack];
   uint8_t bits[kBigStack], flip[kBigStack];
+  uint8_t ord[kBigStack];  // the group's entries are still in the order they were collected in
   int top;
   int nmid;                  // subgroups of the level that fit LDS but are too long to rank
   uint16_t mid[kBigBins];
@@ -1700,17 +1741,20 @@ struct BigShared {
 static_assert(kBigBins * 4 <= kLdsEntries * 8, "the counters fit the second LDS buffer");
 static_assert(kBigBins == 2 * kSortThreads, "two counters per thread in the level's scan");
 
+// `bits` of the whole segment is already what differing_bits would find (the caller looked at
+// the entries when it collected them, in index order).
 __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uint32_t m, int bits,
                                                  const SegmentOut &fin, SortShared &sh,
                                                  BigShared &bg, uint64_t *lds_a, uint64_t *lds_b) {
   const int tid = threadIdx.x;
   uint32_t *cnt = reinterpret_cast<uint32_t *>(lds_b);
-  constexpr int kInFlight = 4;  // entries a thread has under way in the passes over global memory
+  constexpr int kInFlight = 8;  // entries a thread has under way in the passes over global memory
   if (tid == 0) {
     bg.off[0] = 0u;
     bg.len[0] = m;
     bg.bits[0] = (uint8_t)bits;
     bg.flip[0] = 0;
+    bg.ord[0] = 1;
     bg.top = 1;
   }
   __syncthreads();
@@ -1720,13 +1764,29 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
     const uint32_t off = bg.off[top - 1], len = bg.len[top - 1];
     int rem = bg.bits[top - 1];
     const bool flip = bg.flip[top - 1] != 0;
+    const bool ordered = bg.ord[top - 1] != 0;
     __syncthreads();
     if (tid == 0) bg.top = top - 1;
     const uint64_t *src = flip ? g1 : g0;
     uint64_t *dst = flip ? g0 : g1;
-    rem = differing_bits(src, off, len, rem, sh);
-    if (rem == 0) {
-      for (uint32_t i = tid; i < len; i += kSortThreads) fin(off + i, src[off + i]);
+    if (!ordered) rem = differing_bits(src, off, len, rem, sh);
+    // Entries that differ in their indices only -- equal priorities -- are in place when they
+    // are still in index order, as collected (the cursors of a level hand out places in the
+    // order the waves come by: below the first level the order is lost).
+    if (rem == 0 || (ordered && rem <= 32)) {
+      for (uint32_t i0 = tid; i0 < len; i0 += kSortThreads * kInFlight) {
+        uint64_t ent[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+          const uint32_t i = i0 + (uint32_t)u * kSortThreads;
+          ent[u] = src[off + (i < len ? i : 0u)];
+        }
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+          const uint32_t i = i0 + (uint32_t)u * kSortThreads;
+          if (i < len) fin(off + i, ent[u]);
+        }
+      }
       __syncthreads();
       continue;
     }
@@ -1741,7 +1801,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
         const uint32_t i = i0 + (uint32_t)u * kSortThreads + tid;
-        ent[u] = i < len ? src[off + i] : 0ull;
+        ent[u] = src[off + (i < len ? i : 0u)];  // (no test around the load; not looked at beyond the end)
       }
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
@@ -1781,7 +1841,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
         const uint32_t i = i0 + (uint32_t)u * kSortThreads + tid;
-        ent[u] = i < len ? src[off + i] : 0ull;
+        ent[u] = src[off + (i < len ? i : 0u)];  // (no test around the load; not looked at beyond the end)
       }
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
@@ -1811,6 +1871,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
             bg.len[at] = bg.gstart[d0 + 1] - cs;
             bg.bits[at] = (uint8_t)shift;
             bg.flip[at] = flip ? 0 : 1;
+            bg.ord[at] = 0;
             bg.top = at + 1;
           }
         } else {
@@ -1888,7 +1949,7 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
   const uint32_t lo_key = bin_lo_key(map, lo_bin);
   const uint32_t hi_key = bin_hi_key(map, hi_bin);
   const bool in_lds = m <= (uint32_t)kLdsEntries;
-  uint32_t *pos_glb = reinterpret_cast<uint32_t *>(buf1 + out_lo);
+  int big_bits = 0;  // of a segment that does not fit LDS: the low bits in which its entries differ
   __syncthreads();
 
   // One pass over the segment ids, then the segment's entries (key, inverted index) are fetched
@@ -1930,12 +1991,12 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
     int nc = 0;
 #pragma unroll
     for (int g = 0; g < kLoads / 4; ++g) nc += __popcll(hits[g]);
-    if (wave_ballot(nc != 0) != 0ull) {
+    if (in_lds && wave_ballot(nc != 0) != 0ull) {
       const int inc = wave_inclusive_sum(nc);
       uint32_t base = 0;
       if (lane == kWave - 1) base = atomicAdd(&s_cur, (uint32_t)inc);
       base = (uint32_t)__builtin_amdgcn_readlane((int)base, kWave - 1) + (uint32_t)(inc - nc);
-      if (in_lds) {
+      {  // (the entries' order in LDS does not matter: they are sorted next)
 #pragma unroll
         for (int g = 0; g < kLoads / 4; ++g) {
           uint64_t h = hits[g];
@@ -1953,8 +2014,11 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
             }
 #pragma unroll
             for (int f = 0; f < kFetch; ++f) {
-              key[f] = pos[f] < kk ? ckey[pos[f]] : 0u;
-              idx[f] = pos[f] < kk ? cidx[pos[f]] : 0u;
+              // (no test around the loads -- the compiler would wait for each one where the paths
+              // meet --: a slot without a hit loads the first entry and does not look at it)
+              const uint32_t at = pos[f] < kk ? pos[f] : 0u;
+              key[f] = ckey[at];
+              idx[f] = cidx[at];
             }
 #pragma unroll
             for (int f = 0; f < kFetch; ++f) {
@@ -1965,46 +2029,72 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
             }
           }
         }
-      } else {
-        // a long segment (thousands of equal priorities): most ids of a lane are hits, and lanes
-        // that each fetched their own would touch a cache line per lane and load.  The
-        // positions go to the second global buffer first and are fetched in their order.
-#pragma unroll
-        for (int g = 0; g < kLoads / 4; ++g) {
-          uint64_t h = hits[g];
-          while (h != 0ull) {
-            const int bit = __builtin_ctzll(h);
-            h &= h - 1ull;
-            if (base < m)
-              pos_glb[base] = ((uint32_t)(g * 4 + (bit >> 4)) * kSortThreads + tid) * 16 + (uint32_t)(bit & 15);
-            ++base;
-          }
-        }
       }
     }
   }
   __syncthreads();
   if (!in_lds) {
-    constexpr int kGathers = 8;
-    for (uint32_t i = tid; i < m; i += kSortThreads * kGathers) {
-      uint32_t pos[kGathers], key[kGathers], idx[kGathers];
+    // A long segment (thousands of equal priorities, or a crowd in a narrow range): most ids are
+    // hits.  A wave takes a stretch of the ids, a lane an id of every 64: the loads of the keys
+    // and indices and the stores of the entries fall side by side, and the entries end up in the
+    // order of the candidate arrays -- index order --, which lets a segment of equal priorities
+    // go to the output as it is.
+    constexpr int kWaves = kSortThreads / kWave;
+    __shared__ uint32_t s_wcnt[kWaves];
+    const int wave = tid >> 6;
+    const uint8_t seg = (uint8_t)blockIdx.x;
+    const uint32_t per_wave = (kk + kWaves * kWave - 1) / (kWaves * kWave) * kWave;
+    const uint32_t w_begin = (uint32_t)wave * per_wave < kk ? (uint32_t)wave * per_wave : kk;
+    const uint32_t w_end = w_begin + per_wave < kk ? w_begin + per_wave : kk;
+    // how many of the wave's ids are hits: sixteen ids per load, the zero bytes of id ^ own id
+    uint32_t cnt = 0;
+    for (uint32_t c = w_begin + (uint32_t)lane * 16u; c < w_end; c += kWave * 16u) {
+      if (c + 16u <= w_end) {
+        const u32x4 ids = *reinterpret_cast<const u32x4 *>(cseg + c);
 #pragma unroll
-      for (int u = 0; u < kGathers; ++u) {
-        const uint32_t iu = i + (uint32_t)u * kSortThreads;
-        pos[u] = iu < m ? pos_glb[iu] : kk;
-      }
-#pragma unroll
-      for (int u = 0; u < kGathers; ++u) {
-        key[u] = pos[u] < kk ? ckey[pos[u]] : 0u;
-        idx[u] = pos[u] < kk ? cidx[pos[u]] : 0u;
-      }
-#pragma unroll
-      for (int u = 0; u < kGathers; ++u) {
-        const uint32_t iu = i + (uint32_t)u * kSortThreads;
-        if (iu < m) buf0[out_lo + iu] = ((uint64_t)(key[u] - lo_key) << 32) | (uint32_t)~idx[u];
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t t = ids[w] ^ pattern;
+          cnt += (uint32_t)__popc(~(((t & 0x7f7f7f7fu) + 0x7f7f7f7fu) | t | 0x7f7f7f7fu));
+        }
+      } else {
+        for (uint32_t e = c; e < w_end; ++e) cnt += cseg[e] == seg ? 1u : 0u;
       }
     }
+    cnt = (uint32_t)wave_sum((int)cnt);
+    if (lane == 0) s_wcnt[wave] = cnt;
     __syncthreads();
+    uint32_t run = (uint32_t)wave_sum((int)(lane < wave ? s_wcnt[lane] : 0u));
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    constexpr int kGathers = 16;
+    uint64_t bits_or = 0ull, bits_and = ~0ull;  // of the entries: which bits differ among them
+    for (uint32_t c0 = w_begin; c0 < w_end; c0 += kWave * kGathers) {
+      uint32_t key[kGathers], idx[kGathers];
+      uint8_t id[kGathers];
+#pragma unroll
+      for (int u = 0; u < kGathers; ++u) {
+        // (loads without a test around them, see above: beyond the stretch's end its last id
+        // is loaded once more and not looked at)
+        const uint32_t c = c0 + (uint32_t)u * kWave + lane;
+        const uint32_t at = c < w_end ? c : w_end - 1u;
+        id[u] = cseg[at];
+        key[u] = ckey[at];
+        idx[u] = cidx[at];
+      }
+#pragma unroll
+      for (int u = 0; u < kGathers; ++u) {
+        const bool hit = c0 + (uint32_t)u * kWave + lane < w_end && id[u] == seg;
+        const uint64_t b = wave_ballot(hit);
+        const uint32_t place = run + (uint32_t)__popcll(b & lt_mask);
+        if (hit && place < m) {
+          const uint64_t ent = ((uint64_t)(key[u] - lo_key) << 32) | (uint32_t)~idx[u];
+          buf0[out_lo + place] = ent;
+          bits_or |= ent;
+          bits_and &= ent;
+        }
+        run += (uint32_t)__popcll(b);
+      }
+    }
+    big_bits = differing_bits_of(bits_or, bits_and, 64, sh);  // (ends with a barrier)
   }
 
   // An entry holds its key as the distance from the segment's smallest possible key: the bits
@@ -2018,7 +2108,8 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
   if (in_lds)
     sort_segment(lds_a, lds_b, m, bits, out, sh);
   else
-    sort_big_segment(buf0 + out_lo, buf1 + out_lo, m, bits, out, sh, bg, lds_a, lds_b);
+    sort_big_segment(buf0 + out_lo, buf1 + out_lo, m, big_bits < bits ? big_bits : bits, out, sh, bg,
+                     lds_a, lds_b);
 }
 static_assert(kSortThreads >= kSortBins, "a thread per digit in the segment sort's scan");
 
