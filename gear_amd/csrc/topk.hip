@@ -1729,6 +1729,7 @@ __device__ __forceinline__ void sort_segment(uint64_t *a, uint64_t *b, uint32_t 
 // down another level.  The level's counters live in the second LDS buffer, which is idle then.
 constexpr int kBigStack = 32;
 constexpr int kBigBits = 11, kBigBins = 1 << kBigBits;
+constexpr int kBigSubgroups = 16;
 struct BigShared {
   uint32_t gstart[kBigBins + 1];
   uint32_t off[kBigStack], len[kBigStack];
@@ -1737,9 +1738,54 @@ struct BigShared {
   int top;
   int nmid;                  // subgroups of the level that fit LDS but are too long to rank
   uint16_t mid[kBigBins];
+  int nbig;                  // subgroups of the level that exceed LDS (a group in index order only)
+  uint16_t big[kBigSubgroups];
 };
+static_assert((kBucketMaxK + kLdsEntries - 1) / kLdsEntries <= kBigSubgroups,
+              "every subgroup of a segment that exceeds LDS has a slot");
 static_assert(kBigBins * 4 <= kLdsEntries * 8, "the counters fit the second LDS buffer");
 static_assert(kBigBins == 2 * kSortThreads, "two counters per thread in the level's scan");
+
+// The entries of src[0, len) for which pred holds go to dst[0, ...) in the order they have in
+// src: a wave takes a stretch of src, counts its hits, and once the counts of the waves before
+// it are known, copies them -- a lane an entry of every 64, so that loads and stores fall side
+// by side.  Returns nothing; wcnt: a word per wave in LDS.  Called by every thread of the workgroup.
+template <typename P>
+__device__ __forceinline__ void ordered_compact(const uint64_t *src, uint32_t len, uint64_t *dst,
+                                                P pred, uint32_t *wcnt) {
+  constexpr int kWaves = kSortThreads / kWave;
+  constexpr int kLoadsAhead = 8;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t per_wave = (len + kWaves * kWave - 1) / (kWaves * kWave) * kWave;
+  const uint32_t w_begin = (uint32_t)wave * per_wave < len ? (uint32_t)wave * per_wave : len;
+  const uint32_t w_end = w_begin + per_wave < len ? w_begin + per_wave : len;
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  uint32_t run = 0;
+  for (int pass = 0; pass < 2; ++pass) {
+    for (uint32_t c0 = w_begin; c0 < w_end; c0 += kWave * kLoadsAhead) {
+      uint64_t ent[kLoadsAhead];
+#pragma unroll
+      for (int u = 0; u < kLoadsAhead; ++u) {
+        // (no test around the load; beyond the stretch its last entry, not looked at)
+        const uint32_t c = c0 + (uint32_t)u * kWave + lane;
+        ent[u] = src[c < w_end ? c : w_end - 1u];
+      }
+#pragma unroll
+      for (int u = 0; u < kLoadsAhead; ++u) {
+        const bool hit = c0 + (uint32_t)u * kWave + lane < w_end && pred(ent[u]);
+        const uint64_t b = wave_ballot(hit);
+        if (pass == 1 && hit) dst[run + (uint32_t)__popcll(b & lt_mask)] = ent[u];
+        run += (uint32_t)__popcll(b);
+      }
+    }
+    if (pass == 0) {
+      if (lane == 0) wcnt[wave] = run;
+      __syncthreads();
+      run = (uint32_t)wave_sum((int)(lane < wave ? wcnt[lane] : 0u));
+    }
+  }
+  __syncthreads();
+}
 
 // `bits` of the whole segment is already what differing_bits would find (the caller looked at
 // the entries when it collected them, in index order).
@@ -1758,6 +1804,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
     bg.top = 1;
   }
   __syncthreads();
+  bool first = true;  // the whole segment: its differing bits are known
   while (true) {
     const int top = bg.top;
     if (top == 0) break;
@@ -1769,10 +1816,13 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
     if (tid == 0) bg.top = top - 1;
     const uint64_t *src = flip ? g1 : g0;
     uint64_t *dst = flip ? g0 : g1;
-    if (!ordered) rem = differing_bits(src, off, len, rem, sh);
+    if (!first) rem = differing_bits(src, off, len, rem, sh);
+    first = false;
     // Entries that differ in their indices only -- equal priorities -- are in place when they
-    // are still in index order, as collected (the cursors of a level hand out places in the
-    // order the waves come by: below the first level the order is lost).
+    // are still in index order, as collected.  (The cursors of a level hand out places in the
+    // order the waves come by: the order is lost there, except for the subgroups that exceed
+    // LDS -- they are few, and they are where thousands of equal priorities end up when other
+    // keys share their segment --, which a group in index order hands on in index order.)
     if (rem == 0 || (ordered && rem <= 32)) {
       for (uint32_t i0 = tid; i0 < len; i0 += kSortThreads * kInFlight) {
         uint64_t ent[kInFlight];
@@ -1823,7 +1873,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
       bg.gstart[2 * tid] = before;
       bg.gstart[2 * tid + 1] = before + c0;
       if (tid == kSortThreads - 1) bg.gstart[kBigBins] = before + c0 + c1;
-      if (tid == 0) bg.nmid = 0;
+      if (tid == 0) bg.nmid = bg.nbig = 0;
       __syncthreads();
       cnt[2 * tid] = before;  // cursors
       cnt[2 * tid + 1] = before + c0;
@@ -1833,8 +1883,19 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
           bg.mid[atomicAdd(&bg.nmid, 1)] = (uint16_t)(2 * tid);
         if (c1 > (uint32_t)kSmallGroup && c1 <= (uint32_t)kLdsEntries)
           bg.mid[atomicAdd(&bg.nmid, 1)] = (uint16_t)(2 * tid + 1);
+        if (ordered && c0 > (uint32_t)kLdsEntries) bg.big[atomicAdd(&bg.nbig, 1)] = (uint16_t)(2 * tid);
+        if (ordered && c1 > (uint32_t)kLdsEntries)
+          bg.big[atomicAdd(&bg.nbig, 1)] = (uint16_t)(2 * tid + 1);
       }
       __syncthreads();
+    }
+    // the subgroups that exceed LDS, in the order the group has them
+    const int nbig = bg.nbig;
+    for (int qb = 0; qb < nbig; ++qb) {
+      const uint32_t b = bg.big[qb];
+      ordered_compact(
+          src + off, len, dst + off + bg.gstart[b],
+          [&](uint64_t e) { return mask - (uint32_t)((e >> shift) & mask) == b; }, sh.wsum);
     }
     for (uint32_t i0 = 0; i0 < len; i0 += kSortThreads * kInFlight) {
       uint64_t ent[kInFlight];
@@ -1845,8 +1906,10 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
       }
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
-        const bool valid = i0 + (uint32_t)u * kSortThreads + tid < len;
-        const uint32_t at = cursor_take(cnt, mask - (uint32_t)((ent[u] >> shift) & mask), valid);
+        const uint32_t d = mask - (uint32_t)((ent[u] >> shift) & mask);
+        bool valid = i0 + (uint32_t)u * kSortThreads + tid < len;
+        for (int qb = 0; qb < nbig; ++qb) valid = valid && d != bg.big[qb];  // (those are in place)
+        const uint32_t at = cursor_take(cnt, d, valid);
         if (valid) dst[off + at] = ent[u];
       }
     }
@@ -1871,7 +1934,7 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
             bg.len[at] = bg.gstart[d0 + 1] - cs;
             bg.bits[at] = (uint8_t)shift;
             bg.flip[at] = flip ? 0 : 1;
-            bg.ord[at] = 0;
+            bg.ord[at] = ordered ? 1 : 0;
             bg.top = at + 1;
           }
         } else {
