@@ -1002,6 +1002,48 @@ def run_scan(args):
                   "traffic": None}, {"yardsticks": yard})
 
 
+TOPK_INPUTS = {
+    "lognormal": "lognormal ** 0.6 (the priorities of every other workload here)",
+    "equal": "all priorities equal",
+    "integers": "integers 0..999 (ten thousand ties per value at n = 1e7)",
+    "ties": "every 166th priority at one value above all others (60 000 ties at n = 1e7)",
+    "ties-neighbours": "the same with a hundred entries a few ulps above the ties",
+    "ascending": "sorted ascending (the selection is the array's end)",
+    "hot-stretch": "k consecutive entries above everything else",
+    "hot-half": "k / 2 consecutive entries above everything else",
+    "misleading": "the 2048 sampled positions hold the largest priorities (the sampled bound fails)",
+}
+
+
+def _topk_input(np, n, k, kind):
+    """The priorities of --workload topk: lognormal, or one of the shapes that take the selection
+    off its usual path (masses of ties, clustered maxima, a sample that misleads)."""
+    rng = np.random.default_rng(7)
+    w = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    if kind == "equal":
+        w[:] = 1.0
+    elif kind == "integers":
+        w = rng.integers(0, 1000, size=n).astype(np.float32)
+    elif kind in ("ties", "ties-neighbours"):
+        w[rng.random(n) < 1.0 / 166.0] = 100.0
+        if kind == "ties-neighbours":
+            at = rng.permutation(n)[:100]
+            w[at] = np.float32(100.0) + np.float32(1e-4) * rng.integers(1, 8, size=100).astype(np.float32)
+    elif kind == "ascending":
+        w.sort()
+    elif kind in ("hot-stretch", "hot-half"):
+        m = k if kind == "hot-stretch" else k // 2
+        a = min(7 * n // 10, n - m)
+        w[a:a + m] += np.float32(100.0)
+    elif kind == "misleading":
+        samples = 2048
+        stride = n // samples
+        s_ = np.arange(samples, dtype=np.uint64)
+        off = (((s_ * np.uint64(2654435761)) & np.uint64(0xffffffff)) * np.uint64(stride)) >> np.uint64(32)
+        w[(s_ * np.uint64(stride) + off).astype(np.int64)] = (1000.0 + np.arange(samples)).astype(np.float32)
+    return w
+
+
 def run_topk(args):
     """One kernel chain on its own: top --k of --n fp32 priorities (--topk-order value|index)."""
     import numpy as np
@@ -1009,8 +1051,7 @@ def run_topk(args):
     from gear_amd import ops
     n, k = args.n, args.k
     by_value = args.topk_order == "value"
-    rng = np.random.default_rng(7)
-    pri = torch.from_numpy((rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)).cuda()
+    pri = torch.from_numpy(_topk_input(np, n, k, args.topk_input)).cuda()
     if args.calibrate_copy:
         _calibrate_copy(torch, ops)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
@@ -1054,8 +1095,8 @@ def run_topk(args):
             "what": "HIP events around back-to-back launches, same n and k; torch.topk is the "
                     "library selection, pri.sum() one read of the priorities (two launches)"}
     return _line(n / (ms * 1e-3), "priorities/s", args, ms,
-                 "topk: top %d of %d fp32 priorities, ordered by %s%s" %
-                 (k, n, args.topk_order, ", warm calls" if args.topk_warm else ""),
+                 "topk: top %d of %d fp32 priorities (%s), ordered by %s%s" %
+                 (k, n, args.topk_input, args.topk_order, ", warm calls" if args.topk_warm else ""),
                  {"bound": "hbm", "kernel": "top-k chain (prep, level0, member_hist x2, count, "
                                             "write" + (", segment_sort)" if by_value else ")"),
                   "achieved": alg / (avg * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -1082,6 +1123,9 @@ def main():
     ap.add_argument("--hostlink-trajectories", type=int, default=150,
                     help="config4: trajectories (28.2 MB each) of the pinned table of that sub-record")
     ap.add_argument("--topk-order", default="value", choices=["value", "index"])
+    ap.add_argument("--topk-input", default="lognormal", choices=sorted(TOPK_INPUTS),
+                    help="topk: the shape of the priorities; " +
+                         "; ".join("%s = %s" % kv for kv in sorted(TOPK_INPUTS.items())))
     ap.add_argument("--topk-warm", action="store_true",
                     help="topk: calls after the first take up the previous call's bound")
     ap.add_argument("--trajectories3", type=int, default=100_000,

@@ -2229,9 +2229,10 @@ int topk_launch(const float *priorities, int64_t n, int64_t k, int sorted_by_val
   const Geom g = geom(n, k);
 
   // The hint: rank of the sample that safely lies below the k-th largest priority -- the sample's
-  // expected share of k plus six standard deviations and a little.  No sample when the lists hold
-  // whole ranges anyway, when the input is small, or when k is a large part of it (the lists
-  // would hold most of the input: the levels stream instead).
+  // expected share of k plus six standard deviations and a little.  No sample when the input is
+  // small or when k is a large part of it (the lists would hold most of the input: the levels
+  // stream instead).  (Lists that hold whole ranges cannot overflow; with a sample they hold the
+  // candidates only, and the launches after level 0 walk a tenth of the input instead of all.)
   const int list_all = g.list_cap >= g.wave_len ? 1 : 0;
   uint32_t rank = 0;
   // Samples per thread: the fewest with which the entries above the hint fit a wave's list with
@@ -2253,7 +2254,7 @@ int topk_launch(const float *priorities, int64_t n, int64_t k, int sorted_by_val
   int per = 2;
   while (per < kMaxSamplesPerThread && !lists_hold(per)) per *= 4;
   while (per > 2 && n < 128 * (int64_t)per * kThreads) per /= 4;  // strides of 128 elements or more
-  if (!list_all && lists_hold(per) && n >= 128 * (int64_t)per * kThreads && k <= n / 16 &&
+  if ((list_all || lists_hold(per)) && n >= 128 * (int64_t)per * kThreads && k <= n / 8 &&
       env_int("GEAR_HIP_TOPK_HINT", 1) != 0) {
     const double r = hint_rank(per);
     if (r < (double)per * kThreads / 4) rank = (uint32_t)r + 1u;

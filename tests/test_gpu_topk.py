@@ -267,6 +267,29 @@ def test_topk_with_a_misleading_sample(oracle):
     _check_topk(oracle, ops, neg, 30_000, "all negative")
 
 
+def test_topk_small_inputs_with_a_sample(oracle):
+    """Inputs of a few hundred thousand priorities: a wave's list is as long as its range (it
+    cannot overflow), and the sample still decides which entries are listed -- up to k = n / 8."""
+    from gear_amd import ops
+    rng = np.random.default_rng(97)
+    for n, k in ((262_144, 1), (300_000, 37_500), (600_000, 65_536), (1_000_000, 125_000),
+                 (1_000_000, 125_001)):
+        base = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+        _check_topk(oracle, ops, base, k, "lognormal")
+        ties = base.copy()
+        ties[rng.permutation(n)[:max(1, k - k // 8)]] = np.float32(base.max())
+        _check_topk(oracle, ops, ties, k, "most of the selection at the maximum")
+        hot = base.copy()
+        hot[n // 3:n // 3 + max(1, k // 2)] += np.float32(50.0)
+        _check_topk(oracle, ops, hot, k, "a hot stretch")
+        if k > 1:
+            high = base.copy()
+            pos = _sampled_positions(n, _sample_size(n, k))
+            high[pos] = 1000.0 + rng.random(pos.size, dtype=np.float32)
+            _check_topk(oracle, ops, high, k, "sample overstates")
+    _check_topk(oracle, ops, np.full(500_000, 1.5, np.float32), 50_000, "all equal")
+
+
 def _check_state(oracle, state, w, k, by_value, label):
     announce("warm topk %s n=%d k=%d by_value=%d" % (label, len(w), k, by_value))
     vals, idx = state.select(_dev(w), k, sorted_by_value=by_value)
