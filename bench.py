@@ -665,9 +665,8 @@ def run_config3(args):
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(args.steps)]
 
-    # length-weighted draw, then sort + length look-up in one launch, the start offsets, and the
-    # gather through a plan made once (same batch tensors every step)
-    pos = torch.empty(B, dtype=torch.int64, device="cuda")
+    # length-weighted draw, sort, length look-up and window starts in one launch, and the gather
+    # through a plan made once (same batch tensors every step)
     traj = torch.empty(B, dtype=torch.int64, device="cuda")
     loc = torch.empty(B, dtype=torch.int64, device="cuda")
     lens = torch.empty(B, dtype=torch.int64, device="cuda")
@@ -675,11 +674,11 @@ def run_config3(args):
     plan = ops.GatherPlan(table, tab.traj_stride, cols, B)
 
     def select(ua, ub):
+        # length-weighted trajectories, sorted, their lengths and the window starts
+        # floor(ub * (len - span + 1)): one launch after the prefix sum
         ops.prefix_sum_i64(lengths, out=prefix)
-        ops.upper_bound_i64(prefix, ua, unit_uniforms=True, idx_out=pos)
-        ops.sort_lookup(pos, tab.capacity, lengths_table=lengths, sampled_out=traj, local_out=loc,
-                        lens_out=lens)
-        start.copy_(ub * (lens - (span - 1)))   # synthetic start offsets (an input of the config)
+        ops.sample_lookup(prefix, ua, lengths_table=lengths, sampled_out=traj, local_out=loc,
+                          lens_out=lens, start_uniforms=ub, window=span, starts_out=start)
 
     def step(i, slot):
         select(u1[i], u2[i])

@@ -76,6 +76,9 @@ SIGNATURES = {
     "gear_hip_sample_lookup_f64": (c_int, [c_void_p, c_i64, c_void_p, c_i64, c_int, c_void_p, c_i64,
                                            c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_size_t, c_void_p]),
+    "gear_hip_sample_lookup_i64": (c_int, [c_void_p, c_i64, c_void_p, c_i64, c_int, c_void_p, c_i64,
+                                           c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_i64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "gear_hip_sort_lookup_i64": (c_int, [c_void_p, c_i64, c_i64, c_void_p, c_i64, c_i64, c_void_p,
                                          c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                          c_void_p]),

@@ -87,55 +87,100 @@ __global__ __launch_bounds__(kBlock) void normalise_kernel(const double *__restr
   if (j < num) out[j] = (float)(wraw[j] / m);
 }
 
-__global__ __launch_bounds__(kBlock) void search_i64_kernel(const int64_t *__restrict__ prefix,
-                                                            int64_t n, const void *u, int64_t num,
-                                                            int unit,
-                                                            int64_t *__restrict__ idx_out) {
-  const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (j >= num) return;
-  const int64_t total = prefix[n - 1];
-  int64_t t;
-  if (unit)
-    t = (int64_t)floor(static_cast<const double *>(u)[j] * (double)total);
-  else
-    t = static_cast<const int64_t *>(u)[j];
-  int64_t i = upper_bound_dev<int64_t>(prefix, n, t);
-  if (i > n - 1) i = n - 1;
-  idx_out[j] = i;
+// The draw of an int64 prefix (a sampler over lengths): u holds doubles in [0, 1) (unit) or
+// int64 targets.
+struct DrawI64 {
+  const int64_t *prefix;
+  int64_t n;
+  const void *u;
+  int unit;
+  __device__ __forceinline__ int64_t operator()(int64_t j) const {
+    const int64_t total = prefix[n - 1];
+    int64_t t;
+    if (unit)
+      t = (int64_t)floor(static_cast<const double *>(u)[j] * (double)total);
+    else
+      t = static_cast<const int64_t *>(u)[j];
+    const int64_t i = upper_bound_dev<int64_t>(prefix, n, t);
+    return i > n - 1 ? n - 1 : i;
+  }
+};
+// ... of an fp64 prefix: u holds floats, in [0, 1) (unit) or targets.
+struct DrawF64 {
+  const double *prefix;
+  int64_t n;
+  const float *u;
+  int unit;
+  __device__ __forceinline__ int64_t operator()(int64_t j) const {
+    const double total = prefix[n - 1];
+    const double t = unit ? (double)u[j] * total : (double)u[j];
+    const int64_t i = upper_bound_dev<double>(prefix, n, t);
+    return i > n - 1 ? n - 1 : i;
+  }
+};
+
+__global__ __launch_bounds__(kSearchBlock) void search_i64_kernel(DrawI64 draw, int64_t num,
+                                                                  int64_t *__restrict__ idx_out) {
+  const int64_t j = (int64_t)blockIdx.x * kSearchBlock + threadIdx.x;
+  if (j < num) idx_out[j] = draw(j);
 }
 
 // The ranking sort of radix_sort.hpp over the found indices, fused with the split into window
 // arguments.  Used for prefixes shorter than 2^32 entries (the compare key is the index as
 // uint32_t); longer ones take the radix sort.
+struct Split {
+  int64_t *sorted_out;
+  int64_t T, modulo;
+  int64_t *idxs, *tss, *lens;
+  // the entry at sorted place `rank` is the flat index `mine` (below 2^32)
+  __device__ __forceinline__ void operator()(int64_t rank, int64_t f) const {
+    const uint32_t mine = (uint32_t)f;
+    if (sorted_out) sorted_out[rank] = f;
+    if (T > 0) {
+      int64_t traj, ts;
+      if (T <= 0xffffffffll && modulo <= 0xffffffffll) {
+        uint32_t f32 = mine;  // 32-bit division is a fraction of the 64-bit one
+        if (modulo > 0) f32 %= (uint32_t)modulo;
+        const uint32_t q = f32 / (uint32_t)T;
+        traj = q;
+        ts = f32 - q * (uint32_t)T;
+      } else {
+        if (modulo > 0) f %= modulo;
+        traj = f / T;
+        ts = f - traj * T;
+      }
+      idxs[rank] = traj;
+      tss[rank] = ts;
+      if (lens) lens[rank] = ts + 1;
+    }
+  }
+};
+
 __global__ __launch_bounds__(radix::kRankBlock) void rank_split_kernel(
-    const int64_t *__restrict__ raw, int num, int64_t *__restrict__ sorted_out, int64_t T,
-    int64_t modulo, int64_t *__restrict__ idxs, int64_t *__restrict__ tss,
-    int64_t *__restrict__ lens) {
+    const int64_t *__restrict__ raw, int num, Split split) {
   typedef uint32_t K;
   __shared__ radix::RankSmem<K> sm;
   K mine;
   const uint32_t rank = radix::block_rank<K>(sm, num, [&](int j) { return (K)raw[j]; }, &mine);
   const int e = (int)blockIdx.x * kWave + (threadIdx.x & 63);
   if (threadIdx.x >= kWave || e >= num) return;
-  int64_t f = (int64_t)mine;
-  if (sorted_out) sorted_out[rank] = f;
-  if (T > 0) {
-    int64_t traj, ts;
-    if (sizeof(K) == 4 && T <= 0xffffffffll && modulo <= 0xffffffffll) {
-      uint32_t f32 = (uint32_t)mine;  // 32-bit division is a fraction of the 64-bit one
-      if (modulo > 0) f32 %= (uint32_t)modulo;
-      const uint32_t q = f32 / (uint32_t)T;
-      traj = q;
-      ts = f32 - q * (uint32_t)T;
-    } else {
-      if (modulo > 0) f %= modulo;
-      traj = f / T;
-      ts = f - traj * T;
-    }
-    idxs[rank] = traj;
-    tss[rank] = ts;
-    if (lens) lens[rank] = ts + 1;
-  }
+  split((int64_t)rank, (int64_t)mine);
+}
+
+// Search, ranking sort and what follows it in ONE launch, for batches of at most kRankBlock draws
+// (a draw per thread): every workgroup of the ranking sort needs all the found positions, so
+// every one of them runs all the searches itself -- sixteen times the loads for a batch of 1024,
+// out of the caches, in place of a launch and of the round trip of the positions through memory.
+// Draw: DrawF64 or DrawI64; Out: Split or Lookup.
+template <typename Draw, typename Out>
+__global__ __launch_bounds__(radix::kRankBlock) void search_rank_kernel(Draw draw, int num, Out out) {
+  typedef uint32_t K;
+  __shared__ radix::RankSmem<K> sm;
+  K mine;
+  const uint32_t rank = radix::block_rank<K>(sm, num, [&](int j) { return (K)draw(j); }, &mine);
+  const int e = (int)blockIdx.x * kWave + (threadIdx.x & 63);
+  if (threadIdx.x >= kWave || e >= num) return;
+  out((int64_t)rank, (int64_t)mine);
 }
 
 __global__ __launch_bounds__(kBlock) void split_sorted_kernel(const int64_t *__restrict__ flat,
@@ -167,13 +212,23 @@ struct Lookup {
   const int64_t *lengths_table;
   int64_t lengths_n;
   int64_t *sampled, *local, *lens;
+  // a window of `window` steps inside the entry's recorded length, placed by a uniform:
+  // starts[r] = floor(start_u[r] * (length - window + 1)), 0 for a length below the window
+  const double *start_u = nullptr;
+  int64_t window = 0;
+  int64_t *starts = nullptr;
   __device__ __forceinline__ void operator()(int64_t r, int64_t p) const {
     int64_t g = p;
     if (index_table) g = (p >= 0 && p < index_n) ? index_table[p] : 0;
     const int64_t l = g - index_offset;
     if (sampled) sampled[r] = g;
     if (local) local[r] = l;
-    if (lens) lens[r] = (lengths_table && l >= 0 && l < lengths_n) ? lengths_table[l] : 0;
+    const int64_t len = (lengths_table && l >= 0 && l < lengths_n) ? lengths_table[l] : 0;
+    if (lens) lens[r] = len;
+    if (starts) {
+      const int64_t room = len - (window - 1);
+      starts[r] = room > 0 ? (int64_t)floor(start_u[r] * (double)room) : 0;
+    }
   }
 };
 
@@ -262,10 +317,10 @@ extern "C" int gear_hip_upper_bound_i64(const int64_t *prefix, int64_t n, const 
   if (n < 0 || num < 0) return GEAR_HIP_EINVAL;
   if (num == 0) return 0;
   if (n == 0 || !prefix || !u || !idx_out) return GEAR_HIP_EINVAL;
-  const int64_t blocks = ceil_div64(num, kBlock);
+  const int64_t blocks = ceil_div64(num, kSearchBlock);
   if (blocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
-  search_i64_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, as_stream(stream)>>>(
-      prefix, n, u, num, unit_uniforms ? 1 : 0, idx_out);
+  search_i64_kernel<<<dim3((unsigned)blocks), dim3(kSearchBlock), 0, as_stream(stream)>>>(
+      DrawI64{prefix, n, u, unit_uniforms ? 1 : 0}, num, idx_out);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return 0;
 }
@@ -293,12 +348,20 @@ extern "C" int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const
   const int64_t blocks = ceil_div64(num, kBlock);
   const int64_t sblocks = ceil_div64(num, kSearchBlock);
   if (sblocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  const Split split{sorted_out, trajectory_length, modulo, idxs, tss, lens};
+  if (num <= radix::kRankBlock && n < (1ll << 32)) {  // a draw per thread: one launch
+    search_rank_kernel<DrawF64, Split>
+        <<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(
+            DrawF64{prefix, n, u, unit_uniforms ? 1 : 0}, (int)num, split);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
   search_f64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(
       prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   if (num <= radix::kRankMax && n < (1ll << 32)) {
     rank_split_kernel<<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(
-        raw, (int)num, sorted_out, trajectory_length, modulo, idxs, tss, lens);
+        raw, (int)num, split);
     GEARHIP_RETURN_IF_LAUNCH_FAILED();
     return 0;
   }
@@ -321,8 +384,9 @@ namespace {
 
 int check_lookup(const Lookup &look) {
   if (look.index_n < 0 || look.lengths_n < 0) return GEAR_HIP_EINVAL;
-  if (look.lens && !look.lengths_table) return GEAR_HIP_EINVAL;
-  if (!look.sampled && !look.local && !look.lens) return GEAR_HIP_EINVAL;
+  if ((look.lens || look.starts) && !look.lengths_table) return GEAR_HIP_EINVAL;
+  if (look.starts && (!look.start_u || look.window < 1)) return GEAR_HIP_EINVAL;
+  if (!look.sampled && !look.local && !look.lens && !look.starts) return GEAR_HIP_EINVAL;
   return 0;
 }
 
@@ -373,8 +437,54 @@ extern "C" int gear_hip_sample_lookup_f64(const double *prefix, int64_t n, const
   char *ws = static_cast<char *>(workspace);
   int64_t *raw = reinterpret_cast<int64_t *>(ws + w.raw);
   hipStream_t st = as_stream(stream);
+  if (num <= radix::kRankBlock && n < (1ll << 32)) {  // a draw per thread: one launch
+    search_rank_kernel<DrawF64, Lookup>
+        <<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(
+            DrawF64{prefix, n, u, unit_uniforms ? 1 : 0}, (int)num, look);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
   search_f64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(
       prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
+  GEARHIP_RETURN_IF_LAUNCH_FAILED();
+  return sort_and_look_up(raw, num, n, look, ws, w, st);
+}
+
+extern "C" int gear_hip_sample_lookup_i64(const int64_t *prefix, int64_t n, const void *u,
+                                          int64_t num, int unit_uniforms,
+                                          const int64_t *index_table, int64_t index_offset,
+                                          const int64_t *lengths_table, int64_t lengths_n,
+                                          int64_t *sampled_out, int64_t *local_out,
+                                          int64_t *lens_out, const double *start_uniforms,
+                                          int64_t window, int64_t *starts_out, void *workspace,
+                                          size_t workspace_bytes, void *stream) {
+  if (n < 0 || num < 0) return GEAR_HIP_EINVAL;
+  if (num == 0) return 0;
+  if (n == 0 || !prefix || !u) return GEAR_HIP_EINVAL;
+  Lookup look{index_table, n, index_offset, lengths_table, lengths_n, sampled_out, local_out,
+              lens_out};
+  look.start_u = start_uniforms;
+  look.window = window;
+  look.starts = starts_out;
+  int rc = check_lookup(look);
+  if (rc) return rc;
+  const SampleWs w = sample_ws(num);
+  if (!workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 7))
+    return GEAR_HIP_EWORKSPACE;
+  const int64_t sblocks = ceil_div64(num, kSearchBlock);
+  if (sblocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
+  char *ws = static_cast<char *>(workspace);
+  int64_t *raw = reinterpret_cast<int64_t *>(ws + w.raw);
+  hipStream_t st = as_stream(stream);
+  const DrawI64 draw{prefix, n, u, unit_uniforms ? 1 : 0};
+  if (num <= radix::kRankBlock && n < (1ll << 32)) {  // a draw per thread: one launch
+    search_rank_kernel<DrawI64, Lookup>
+        <<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(draw, (int)num,
+                                                                                      look);
+    GEARHIP_RETURN_IF_LAUNCH_FAILED();
+    return 0;
+  }
+  search_i64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(draw, num, raw);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return sort_and_look_up(raw, num, n, look, ws, w, st);
 }

@@ -409,12 +409,28 @@ def _lookup_outputs(num, dev, lengths_table, sampled_out, local_out, lens_out):
 
 
 def sample_lookup(prefix, u, *, unit_uniforms=True, index_table=None, index_offset=0,
-                  lengths_table=None, sampled_out=None, local_out=None, lens_out=None):
+                  lengths_table=None, sampled_out=None, local_out=None, lens_out=None,
+                  start_uniforms=None, window=0, starts_out=None):
     """Weighted draws, sorted, with the loader's look-ups in the same call: positions of the
-    draws in the fp64 prefix, ascending -> (sampled = index_table[position], local = sampled -
-    index_offset, lens = lengths_table[local]).  See gear_hip_sample_lookup_f64."""
-    _need(prefix, torch.float64, "prefix")
-    _need(u, torch.float32, "u")
+    draws in the prefix, ascending -> (sampled = index_table[position], local = sampled -
+    index_offset, lens = lengths_table[local]).  An fp64 prefix takes float32 draws
+    (gear_hip_sample_lookup_f64), an int64 prefix -- a sampler over lengths -- float64 uniforms
+    or int64 targets (gear_hip_sample_lookup_i64); there, `start_uniforms` (float64 in [0, 1), one
+    per draw) and `window` add a fourth result: starts = floor(start_uniforms * (lens - window + 1)),
+    where a window of that many steps begins inside each drawn entry."""
+    if start_uniforms is not None and prefix.dtype != torch.int64:
+        raise ValueError("window starts come with an int64 prefix only")
+    if prefix.dtype == torch.int64:
+        _need(prefix, torch.int64, "prefix")
+        if unit_uniforms:
+            _need(u, torch.float64, "u")
+        else:
+            _need(u, torch.int64, "u")
+        entry = "gear_hip_sample_lookup_i64"
+    else:
+        _need(prefix, torch.float64, "prefix")
+        _need(u, torch.float32, "u")
+        entry = "gear_hip_sample_lookup_f64"
     num, dev = u.numel(), u.device
     if index_table is not None:
         _need(index_table, torch.int64, "index_table")
@@ -424,10 +440,22 @@ def sample_lookup(prefix, u, *, unit_uniforms=True, index_table=None, index_offs
         _need(lengths_table, torch.int64, "lengths_table")
     sampled, local, lens = _lookup_outputs(num, dev, lengths_table, sampled_out, local_out, lens_out)
     ws = _ws.get("sample", _ws_bytes("gear_hip_sample_workspace_bytes", num), dev)
-    call("gear_hip_sample_lookup_f64", _ptr(prefix), prefix.numel(), _ptr(u), num,
-         int(bool(unit_uniforms)), _ptr(index_table), int(index_offset), _ptr(lengths_table),
-         lengths_table.numel() if lengths_table is not None else 0, _ptr(sampled), _ptr(local),
-         _ptr(lens), _ptr(ws), ws.numel(), _stream())
+    args = [_ptr(prefix), prefix.numel(), _ptr(u), num, int(bool(unit_uniforms)), _ptr(index_table),
+            int(index_offset), _ptr(lengths_table),
+            lengths_table.numel() if lengths_table is not None else 0, _ptr(sampled), _ptr(local),
+            _ptr(lens)]
+    starts = None
+    if prefix.dtype == torch.int64:
+        if start_uniforms is not None:
+            _need(start_uniforms, torch.float64, "start_uniforms")
+            if start_uniforms.numel() != num or lengths_table is None or window < 1:
+                raise ValueError("window starts need a uniform per draw, lengths_table and window >= 1")
+            starts = starts_out if starts_out is not None else torch.empty(
+                num, dtype=torch.int64, device=dev)
+        args += [_ptr(start_uniforms), int(window), _ptr(starts)]
+    call(entry, *args, _ptr(ws), ws.numel(), _stream())
+    if starts is not None:
+        return sampled, local, lens, starts
     return sampled, local, lens
 
 

@@ -525,8 +525,8 @@ def test_select_with_lookups_equals_the_separate_calls(oracle):
     of the 4096-entry ranking sort, with an index offset, and against numpy."""
     from gear_amd import ops
     rng = np.random.default_rng(1234)
-    for n, num, offset in ((1, 1, 0), (5_000, 257, 0), (100_000, 4096, 1_000_000),
-                           (100_000, 4097, 77), (1_000_000, 20_000, 5)):
+    for n, num, offset in ((1, 1, 0), (5_000, 257, 0), (300_000, 1024, 3), (300_000, 1025, 3),
+                           (100_000, 4096, 1_000_000), (100_000, 4097, 77), (1_000_000, 20_000, 5)):
         announce("select + look-ups n=%d num=%d offset=%d" % (n, num, offset))
         pri = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
         if n > 10:
@@ -571,6 +571,50 @@ def test_select_with_lookups_equals_the_separate_calls(oracle):
         exp_n = np.where(ok_l, lengths[np.clip(exp_l, 0, n - 1)], 0)
         assert np.array_equal(s4.cpu().numpy(), exp_s) and np.array_equal(l4.cpu().numpy(), exp_l)
         assert np.array_equal(n4.cpu().numpy(), exp_n)
+
+
+def test_select_over_an_int64_prefix_with_window_starts(oracle):
+    """gear_hip_sample_lookup_i64: trajectories drawn by length (int64 prefix, float64 uniforms or
+    int64 targets), sorted, with their lengths and the start of a window inside each --
+    floor(v * (length - window + 1)) -- against the oracle's search and numpy, on both sides of
+    the 1024 draws that one launch searches and ranks, and of the 4096 of the ranking sort."""
+    from gear_amd import ops
+    rng = np.random.default_rng(4242)
+    for n, num, window in ((1, 1, 1), (100_000, 1024, 20), (100_000, 1025, 20), (7_777, 333, 1),
+                           (250_000, 4096, 64), (250_000, 5000, 200)):
+        announce("int64 select + look-ups n=%d num=%d window=%d" % (n, num, window))
+        lengths = rng.integers(1, 1001, size=n).astype(np.int64)
+        if n > 10:
+            lengths[rng.integers(0, n, size=n // 9)] = 0          # never drawn
+        lengths[0] = max(lengths[0], 1)
+        u = rng.random(num)
+        v = rng.random(num)
+        dlen = _dev(lengths)
+        prefix = ops.prefix_sum_i64(dlen)
+        hp = prefix.cpu().numpy()
+        assert np.array_equal(hp, np.cumsum(lengths))
+        traj, local, lens, starts = ops.sample_lookup(prefix, _dev(u), lengths_table=dlen,
+                                                      start_uniforms=_dev(v), window=window)
+        torch.cuda.synchronize()
+        exp = np.sort(oracle.upper_bound_i64(hp, u, unit_uniforms=True))
+        assert np.array_equal(traj.cpu().numpy(), exp)
+        assert np.array_equal(local.cpu().numpy(), exp)
+        assert np.array_equal(lens.cpu().numpy(), lengths[exp])
+        room = lengths[exp] - (window - 1)
+        exp_starts = np.where(room > 0, np.floor(v * room.astype(np.float64)).astype(np.int64), 0)
+        assert np.array_equal(starts.cpu().numpy(), exp_starts)
+        assert np.all(exp_starts + np.minimum(window, lengths[exp]) <= lengths[exp])
+        # int64 targets instead of uniforms, no starts
+        t = rng.integers(0, hp[-1], size=num).astype(np.int64)
+        traj2, _, lens2 = ops.sample_lookup(prefix, _dev(t), unit_uniforms=False, lengths_table=dlen)
+        torch.cuda.synchronize()
+        exp2 = np.sort(np.minimum(np.searchsorted(hp, t, side="right"), n - 1))
+        assert np.array_equal(traj2.cpu().numpy(), exp2)
+        assert np.array_equal(lens2.cpu().numpy(), lengths[exp2])
+    with pytest.raises(ValueError):
+        ops.sample_lookup(ops.prefix_sum(_dev(np.ones(8, np.float32))), _dev(np.zeros(2, np.float32)),
+                          lengths_table=_dev(np.ones(8, np.int64)),
+                          start_uniforms=_dev(np.zeros(2)), window=2)
 
 
 def test_staggered_start_of_the_chained_scan_changes_no_bit():
