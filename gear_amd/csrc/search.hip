@@ -105,20 +105,6 @@ struct DrawI64 {
     return i > n - 1 ? n - 1 : i;
   }
 };
-// ... of an fp64 prefix: u holds floats, in [0, 1) (unit) or targets.
-struct DrawF64 {
-  const double *prefix;
-  int64_t n;
-  const float *u;
-  int unit;
-  __device__ __forceinline__ int64_t operator()(int64_t j) const {
-    const double total = prefix[n - 1];
-    const double t = unit ? (double)u[j] * total : (double)u[j];
-    const int64_t i = upper_bound_dev<double>(prefix, n, t);
-    return i > n - 1 ? n - 1 : i;
-  }
-};
-
 __global__ __launch_bounds__(kSearchBlock) void search_i64_kernel(DrawI64 draw, int64_t num,
                                                                   int64_t *__restrict__ idx_out) {
   const int64_t j = (int64_t)blockIdx.x * kSearchBlock + threadIdx.x;
@@ -165,22 +151,6 @@ __global__ __launch_bounds__(radix::kRankBlock) void rank_split_kernel(
   const int e = (int)blockIdx.x * kWave + (threadIdx.x & 63);
   if (threadIdx.x >= kWave || e >= num) return;
   split((int64_t)rank, (int64_t)mine);
-}
-
-// Search, ranking sort and what follows it in ONE launch, for batches of at most kRankBlock draws
-// (a draw per thread): every workgroup of the ranking sort needs all the found positions, so
-// every one of them runs all the searches itself -- sixteen times the loads for a batch of 1024,
-// out of the caches, in place of a launch and of the round trip of the positions through memory.
-// Draw: DrawF64 or DrawI64; Out: Split or Lookup.
-template <typename Draw, typename Out>
-__global__ __launch_bounds__(radix::kRankBlock) void search_rank_kernel(Draw draw, int num, Out out) {
-  typedef uint32_t K;
-  __shared__ radix::RankSmem<K> sm;
-  K mine;
-  const uint32_t rank = radix::block_rank<K>(sm, num, [&](int j) { return (K)draw(j); }, &mine);
-  const int e = (int)blockIdx.x * kWave + (threadIdx.x & 63);
-  if (threadIdx.x >= kWave || e >= num) return;
-  out((int64_t)rank, (int64_t)mine);
 }
 
 __global__ __launch_bounds__(kBlock) void split_sorted_kernel(const int64_t *__restrict__ flat,
@@ -349,13 +319,6 @@ extern "C" int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const
   const int64_t sblocks = ceil_div64(num, kSearchBlock);
   if (sblocks >= 0x7fffffffll) return GEAR_HIP_ERANGE;
   const Split split{sorted_out, trajectory_length, modulo, idxs, tss, lens};
-  if (num <= radix::kRankBlock && n < (1ll << 32)) {  // a draw per thread: one launch
-    search_rank_kernel<DrawF64, Split>
-        <<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(
-            DrawF64{prefix, n, u, unit_uniforms ? 1 : 0}, (int)num, split);
-    GEARHIP_RETURN_IF_LAUNCH_FAILED();
-    return 0;
-  }
   search_f64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(
       prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
@@ -437,13 +400,6 @@ extern "C" int gear_hip_sample_lookup_f64(const double *prefix, int64_t n, const
   char *ws = static_cast<char *>(workspace);
   int64_t *raw = reinterpret_cast<int64_t *>(ws + w.raw);
   hipStream_t st = as_stream(stream);
-  if (num <= radix::kRankBlock && n < (1ll << 32)) {  // a draw per thread: one launch
-    search_rank_kernel<DrawF64, Lookup>
-        <<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(
-            DrawF64{prefix, n, u, unit_uniforms ? 1 : 0}, (int)num, look);
-    GEARHIP_RETURN_IF_LAUNCH_FAILED();
-    return 0;
-  }
   search_f64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(
       prefix, n, u, num, unit_uniforms ? 1 : 0, raw, nullptr, 0.0, nullptr, nullptr);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
@@ -477,13 +433,6 @@ extern "C" int gear_hip_sample_lookup_i64(const int64_t *prefix, int64_t n, cons
   int64_t *raw = reinterpret_cast<int64_t *>(ws + w.raw);
   hipStream_t st = as_stream(stream);
   const DrawI64 draw{prefix, n, u, unit_uniforms ? 1 : 0};
-  if (num <= radix::kRankBlock && n < (1ll << 32)) {  // a draw per thread: one launch
-    search_rank_kernel<DrawI64, Lookup>
-        <<<dim3((unsigned)ceil_div64(num, kWave)), dim3(radix::kRankBlock), 0, st>>>(draw, (int)num,
-                                                                                      look);
-    GEARHIP_RETURN_IF_LAUNCH_FAILED();
-    return 0;
-  }
   search_i64_kernel<<<dim3((unsigned)sblocks), dim3(kSearchBlock), 0, st>>>(draw, num, raw);
   GEARHIP_RETURN_IF_LAUNCH_FAILED();
   return sort_and_look_up(raw, num, n, look, ws, w, st);

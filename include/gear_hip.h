@@ -277,9 +277,8 @@ int gear_hip_upper_bound_f64(const double *prefix, int64_t n, const float *u, in
  * reference returns, torch.sort(...).values, gear/sampler/global_sampler.py:131,172,195-199 --
  * and, when trajectory_length > 0, split like gear_hip_split_step_index into idxs/tss/lens
  * (lens may be NULL).  sorted_out may be NULL when trajectory_length > 0.
- * Up to 1024 draws take ONE launch (every workgroup of the ranking sort searches the draws
- * itself, a draw per thread), up to 4096 two (search over many workgroups, then the ranking
- * sort, which also splits); larger batches use the multi-pass radix sort.
+ * Up to 4096 draws take two launches (search over many workgroups, then the ranking sort,
+ * which also splits); larger batches use the multi-pass radix sort.
  * workspace: gear_hip_sample_workspace_bytes(num) bytes on the device. */
 size_t gear_hip_sample_workspace_bytes(int64_t num);
 int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const float *u, int64_t num,
@@ -298,8 +297,8 @@ int gear_hip_sample_sorted_f64(const double *prefix, int64_t n, const float *u, 
  * torch.sort(concat_indices[draws]) (gear/sampler/global_sampler.py:131,172,196),
  * indices - index_offset and iset.timesteps[indices.cpu()] on the host
  * (gear/loader/offline_loader.py:161-177): up to 4096 positions take ONE launch after the search
- * (the ranking sort does the look-ups of the entry it places; up to 1024 draws it does the
- * search too), more take the radix sort and an element-wise launch.
+ * (the ranking sort does the look-ups of the entry it places), more take the radix sort and an
+ * element-wise launch.
  *   gear_hip_sample_lookup_f64  positions = upper_bound of the draws u in the fp64 prefix, as
  *                               gear_hip_upper_bound_f64 (index_table, when given, has n entries)
  *   gear_hip_sample_lookup_i64  the same in an int64 prefix (a sampler over lengths), u as for

@@ -577,7 +577,7 @@ def test_select_over_an_int64_prefix_with_window_starts(oracle):
     """gear_hip_sample_lookup_i64: trajectories drawn by length (int64 prefix, float64 uniforms or
     int64 targets), sorted, with their lengths and the start of a window inside each --
     floor(v * (length - window + 1)) -- against the oracle's search and numpy, on both sides of
-    the 1024 draws that one launch searches and ranks, and of the 4096 of the ranking sort."""
+    the 4096 draws of the ranking sort."""
     from gear_amd import ops
     rng = np.random.default_rng(4242)
     for n, num, window in ((1, 1, 1), (100_000, 1024, 20), (100_000, 1025, 20), (7_777, 333, 1),
