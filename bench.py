@@ -990,7 +990,7 @@ def run_scan(args):
     forced = os.environ.get("GEAR_HIP_SCAN_SINGLE_PASS", "")
     ranges = -(-n // 8192)     # what the library does at this size: see gear_amd/csrc/scan.hip
     by_size = ("three launches (range sums, their prefix, scan)" if ranges > 16384 else
-               "two launches" if ranges > 4096 or forced == "0" else "chained single pass")
+               "two launches" if ranges > 8192 or forced == "0" else "chained single pass")
     variant = by_size + (" (default)" if forced == "" else "")
     return _line(n / (ms * 1e-3), "priorities/s", args, ms,
                  "scan: fp64 prefix sum of %d fp32 priorities, %s" % (n, variant),

@@ -4,7 +4,8 @@
 // granules of its range, adds them up in order, and one DPP wave scan per range joins the
 // threads (a wave-private LDS row turns the row-major order of the memory instructions, 1 KiB of
 // consecutive addresses per wave and instruction, into that blocked order and back):
-//  * chained single pass, up to 4096 ranges: scan_ranges_kernel<kChained>.  A workgroup
+//  * chained single pass, up to 4096 ranges (of up to 16384 fp32 elements: 67 M):
+//    scan_ranges_kernel<kChained>.  A workgroup
 //    keeps its range in registers, publishes the range's sum and adds the sums of ALL earlier
 //    ranges (fixed order: bit-reproducible), then writes the prefix: the input is read once.
 //    Range r belongs to workgroup r (no ticket).  A published sum travels as three 64-bit words
@@ -645,12 +646,14 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
     }
     if (cap != hipStreamCaptureStatusNone) chained = false;
   }
-  // Ranges of 2, 4 or 8 granules per thread (2048, 4096 or 8192 fp32 elements): 2 while that
-  // leaves at most 256 ranges, 4 up to 512 ranges, else 8 (a workgroup adds up ALL earlier sums, so
-  // more ranges cost more than they gain once every CU has work).  The chained kernel and the two
-  // launches cut the input the same way, so a rescan finds the sums of the last full scan.
+  // Ranges of 2, 4, 8 or 16 granules per thread (2048 to 16384 fp32 elements): 2 while that
+  // leaves at most 256 ranges, 4 up to 512 ranges, then 8 (a workgroup adds up ALL earlier sums, so
+  // more ranges cost more than they gain once every CU has work), and 16 -- 190 registers, two
+  // workgroups per CU -- where 8 would need more than 4096 ranges (33.5 to 67 M fp32: one read
+  // instead of two, 187 -> 148 us at 6e7).  The chained kernel and the two launches cut the input
+  // the same way, so a rescan finds the sums of the last full scan.
   // Beyond 4096 ranges the words to poll outweigh the second read: two launches, up to 16384
-  // ranges.  (8-byte elements: ranges of 2 granules would be smaller than the 2048 elements the
+  // ranges of 8 granules.  (8-byte elements: ranges of 2 granules would be smaller than the 2048 elements the
   // workspace is laid out for, so they start at 4.)
   constexpr int64_t g1 = (int64_t)kBlock * VE;  // elements per range and granule
   if (VE == 4 && ceil_div64(n, 2 * g1) <= 256)
@@ -659,6 +662,8 @@ int launch_scan(const In *in, Out *out, int64_t n, void *ws, size_t ws_bytes, hi
     return launch_ranges<In, Acc, Out, VE, 4>(in, out, n, ws, st, chained, first_changed);
   else if (ceil_div64(n, 8 * g1) <= kMaxRanges)
     return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, chained, first_changed);
+  else if (ceil_div64(n, 16 * g1) <= kMaxRanges)
+    return launch_ranges<In, Acc, Out, VE, 16>(in, out, n, ws, st, chained, first_changed);
   return launch_ranges<In, Acc, Out, VE, 8>(in, out, n, ws, st, false, first_changed);
 }
 

@@ -178,7 +178,7 @@ int gear_hip_take_i64(const int64_t *table, int64_t n, const int64_t *idx, int64
 
 /* Inclusive prefix sum of fp32 priorities accumulated and written in fp64:
  *     out[i] = sum_{j<=i} (double) in[j]
- * One pass over the input for up to 4096 ranges (n <= 33.5 M): every workgroup publishes the sum
+ * One pass over the input for up to 4096 ranges (n <= 67.1 M): every workgroup publishes the sum
  * of its range and adds the sums of all earlier ranges, with a bounded wait (a workgroup that
  * waited too long sums the missing range itself and publishes it: same bits, no kernel can
  * hang).  Two launches (range sums, then the scan) beyond that, for a stream under graph capture,

@@ -12,10 +12,11 @@ torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
 
 # small sizes, then the sizes at which the range geometry, the staggered start, the streaming
-# loads and the variant change (524 288, 2 097 152, 4 194 304, 16 777 216, 33 554 432, 134 217 728)
+# loads and the variant change (524 288, 2 097 152, 4 194 304, 16 777 216, 33 554 432, 67 108 864,
+# 134 217 728)
 SIZES = [1, 2, 3, 63, 64, 65, 255, 1023, 2047, 2048, 2049, 4095, 4096, 4097, 8191, 8192, 8193,
          100_000, 524_288, 524_289, 1_000_000, 2_097_153, 4_194_305, 10_000_003, 16_777_217,
-         33_554_433, 34_000_001, 134_300_000]
+         33_554_433, 34_000_001, 67_108_864, 67_108_865, 134_300_000]
 
 
 @pytest.fixture(params=["two_launch", "single_pass"])
@@ -419,7 +420,7 @@ def test_chained_scan_ignores_what_the_workspace_held():
             assert torch.equal(scan(), expect), what
 
 
-@pytest.mark.parametrize("n", [4097, 1_000_000, 3_000_001])
+@pytest.mark.parametrize("n", [4097, 1_000_000, 3_000_001, 40_000_001])
 def test_chained_scan_with_no_patience_sums_the_missing_ranges_itself(oracle, n):
     """The chained kernel waits a bounded number of polls for an earlier range's sum and then sums
     that range itself.  With a limit of 0 polls (forced from the host) every workgroup takes
