@@ -1971,6 +1971,92 @@ __device__ __forceinline__ void sort_big_segment(uint64_t *g0, uint64_t *g1, uin
   }
 }
 
+// A segment that exceeds LDS is most often thousands of EQUAL priorities (fresh transitions at the
+// maximum priority, integer returns): its entries then only have to go to the output in index
+// order, which is the order of the candidate arrays, and the workgroups that own no segment in
+// such a call -- its output stretches lie inside the long segment's -- can share that: workgroup
+// `slot` of `parts` stores the entries whose place among the segment's lies in its part.  Every
+// one of them works out alone whether the keys are equal (one pass over the segment's ids and
+// keys: nobody waits for anybody), so they all decide alike.  Returns false, with nothing
+// stored, when the keys differ.  Called by every thread of the workgroup.
+__device__ __forceinline__ bool store_equal_segment(uint32_t seg_id, uint32_t m, uint32_t slot,
+                                                    uint32_t parts, uint32_t kk,
+                                                    const uint32_t *__restrict__ ckey,
+                                                    const uint32_t *__restrict__ cidx,
+                                                    const uint8_t *__restrict__ cseg,
+                                                    const SegmentOut &out, SortShared &sh) {
+  constexpr int kWaves = kSortThreads / kWave;
+  constexpr int kLoadsAhead = 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint8_t seg = (uint8_t)seg_id;
+  const uint32_t per_wave = (kk + kWaves * kWave - 1) / (kWaves * kWave) * kWave;
+  const uint32_t w_begin = (uint32_t)wave * per_wave < kk ? (uint32_t)wave * per_wave : kk;
+  const uint32_t w_end = w_begin + per_wave < kk ? w_begin + per_wave : kk;
+  if (tid < 4) sh.bits_or_and[tid] = tid < 2 ? 0u : 0xffffffffu;
+  __syncthreads();
+  uint32_t cnt = 0, k_or = 0u, k_and = 0xffffffffu;
+  for (uint32_t c0 = w_begin; c0 < w_end; c0 += kWave * kLoadsAhead) {
+    uint8_t id[kLoadsAhead];
+    uint32_t key[kLoadsAhead];
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u) {
+      // (no test around the loads; beyond the stretch its last id once more, not looked at)
+      const uint32_t c = c0 + (uint32_t)u * kWave + lane;
+      const uint32_t at = c < w_end ? c : w_end - 1u;
+      id[u] = cseg[at];
+      key[u] = ckey[at];
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u) {
+      const bool hit = c0 + (uint32_t)u * kWave + lane < w_end && id[u] == seg;
+      cnt += hit ? 1u : 0u;
+      k_or |= hit ? key[u] : 0u;
+      k_and &= hit ? key[u] : 0xffffffffu;
+    }
+  }
+  cnt = (uint32_t)wave_sum((int)cnt);
+  for (int d = 32; d >= 1; d >>= 1) {
+    k_or |= (uint32_t)__shfl_xor((int)k_or, d, kWave);
+    k_and &= (uint32_t)__shfl_xor((int)k_and, d, kWave);
+  }
+  if (lane == 0) {
+    sh.wsum[wave] = cnt;
+    atomicOr(&sh.bits_or_and[0], k_or);
+    atomicAnd(&sh.bits_or_and[2], k_and);
+  }
+  __syncthreads();
+  const uint32_t key = sh.bits_or_and[0];
+  const bool equal = key == sh.bits_or_and[2];
+  uint32_t run = (uint32_t)wave_sum((int)(lane < wave ? sh.wsum[lane] : 0u));
+  __syncthreads();  // (sh is used again by whoever goes on)
+  if (!equal) return false;
+  const uint32_t part_lo = (uint32_t)((uint64_t)m * slot / parts);
+  const uint32_t part_hi = (uint32_t)((uint64_t)m * (slot + 1u) / parts);
+  if (run + cnt <= part_lo || run >= part_hi) return true;  // none of the wave's entries
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  const uint64_t key_part = (uint64_t)(key - out.key_base) << 32;
+  for (uint32_t c0 = w_begin; c0 < w_end; c0 += kWave * kLoadsAhead) {
+    uint8_t id[kLoadsAhead];
+    uint32_t idx[kLoadsAhead];
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u) {
+      const uint32_t c = c0 + (uint32_t)u * kWave + lane;
+      const uint32_t at = c < w_end ? c : w_end - 1u;
+      id[u] = cseg[at];
+      idx[u] = cidx[at];
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u) {
+      const bool hit = c0 + (uint32_t)u * kWave + lane < w_end && id[u] == seg;
+      const uint64_t b = wave_ballot(hit);
+      const uint32_t place = run + (uint32_t)__popcll(b & lt_mask);
+      if (hit && place >= part_lo && place < part_hi) out(place, key_part | (uint32_t)~idx[u]);
+      run += (uint32_t)__popcll(b);
+    }
+  }
+  return true;
+}
+
 __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
     const float *__restrict__ p, int64_t n, int64_t k, const State *state,
     const uint32_t *__restrict__ seg_table, const uint32_t *__restrict__ ckey,
@@ -1996,23 +2082,84 @@ __global__ __launch_bounds__(kSortThreads) void segment_sort_kernel(
   }
   // this workgroup's segment: its bins (highest + 1, kBins0 - lowest; 0 = none) and its stretch
   // of the output, one load; the entries equal to the threshold are not part of any segment
-  const u32x4 mine4 = *reinterpret_cast<const u32x4 *>(seg_table + 4 * blockIdx.x);
+  u32x4 mine4 = *reinterpret_cast<const u32x4 *>(seg_table + 4 * blockIdx.x);
   const uint32_t need_eq = state->k_rem[2];
   const BinMap map = state->map;
   if (tid == 0) s_cur = 0u;
-  const uint32_t hi1 = mine4[0], loinv = mine4[1];
-  if (hi1 == 0u || loinv == 0u) return;
-  const uint32_t hi_bin = hi1 - 1u, lo_bin = (uint32_t)kBins0 - loinv;
-  const uint32_t out_lo = ~mine4[2];
-  uint32_t out_hi = mine4[3];
-  if (out_hi > kk - need_eq) out_hi = kk - need_eq;
-  if (out_lo >= out_hi) return;
-  const uint32_t m = out_hi - out_lo;
+  // How long a segment's stretch of the output is (0: the workgroup owns none).
+  const auto stretch = [&](const u32x4 &e, uint32_t *lo) {
+    uint32_t hi = e[3] > kk - need_eq ? kk - need_eq : e[3];
+    *lo = ~e[2];
+    return (e[0] != 0u && e[1] != 0u && *lo < hi) ? hi - *lo : 0u;
+  };
+  uint32_t out_lo;
+  uint32_t m = stretch(mine4, &out_lo);
+  uint32_t seg_id = blockIdx.x, slot = 0u, parts = 1u;
+  // The workgroups that own no segment, and the owners of segments that exceed LDS, look at the
+  // whole table: which segments are long, which workgroups idle.  The idle ones are dealt out to
+  // the long segments (see store_equal_segment).  (The others have no use for it: a barrier and a
+  // walk over the table cost them a microsecond.)
+  static_assert(kMaxBlocks <= kSortThreads && kMaxBlocks % kWave == 0, "a thread per table entry");
+  __shared__ uint64_t s_long[kMaxBlocks / kWave], s_idle[kMaxBlocks / kWave];
+  if (m == 0u || m > (uint32_t)kLdsEntries) {
+    if (tid < kMaxBlocks) {
+      const u32x4 e = *reinterpret_cast<const u32x4 *>(seg_table + 4 * tid);
+      uint32_t lo;
+      const uint32_t mt = tid < (int)gridDim.x ? stretch(e, &lo) : 0u;
+      const uint64_t lm = wave_ballot(mt > (uint32_t)kLdsEntries), im = wave_ballot(mt == 0u);
+      if (lane == 0) {
+        s_long[tid >> 6] = lm;
+        s_idle[tid >> 6] = im;
+      }
+    }
+    __syncthreads();
+    uint32_t nlong = 0u, nidle = 0u, long_before = 0u, idle_before = 0u;
+#pragma unroll
+    for (int w = 0; w < kMaxBlocks / kWave; ++w) {
+      const uint64_t lm = s_long[w], im = s_idle[w];
+      nlong += (uint32_t)__popcll(lm);
+      nidle += (uint32_t)__popcll(im);
+      if (w * kWave < (int)blockIdx.x) {
+        const int below = (int)blockIdx.x - w * kWave;
+        const uint64_t mask = below >= kWave ? ~0ull : ((1ull << below) - 1ull);
+        long_before += (uint32_t)__popcll(lm & mask);
+        idle_before += (uint32_t)__popcll(im & mask);
+      }
+    }
+    if (m == 0u) {
+      if (nlong == 0u) return;
+      // the idle workgroup's long segment: number idle_before mod nlong of them
+      const uint32_t which = idle_before % nlong;
+      slot = 1u + idle_before / nlong;
+      uint32_t seen = 0u;
+#pragma unroll
+      for (int w = 0; w < kMaxBlocks / kWave; ++w) {
+        uint64_t lm = s_long[w];
+        while (lm != 0ull) {
+          const int bit = __builtin_ctzll(lm);
+          lm &= lm - 1ull;
+          if (seen == which) seg_id = (uint32_t)(w * kWave + bit);
+          ++seen;
+        }
+      }
+      long_before = which;
+      mine4 = *reinterpret_cast<const u32x4 *>(seg_table + 4 * seg_id);
+      m = stretch(mine4, &out_lo);
+    }
+    if (m > (uint32_t)kLdsEntries)  // the segment's owner and the idle workgroups dealt to it
+      parts = 1u + (nidle > long_before ? (nidle - 1u - long_before) / nlong + 1u : 0u);
+  }
+  const uint32_t hi_bin = mine4[0] - 1u, lo_bin = (uint32_t)kBins0 - mine4[1];
   // keys of the segment lie inside the bins' key range
   const uint32_t lo_key = bin_lo_key(map, lo_bin);
   const uint32_t hi_key = bin_hi_key(map, hi_bin);
   const bool in_lds = m <= (uint32_t)kLdsEntries;
   int big_bits = 0;  // of a segment that does not fit LDS: the low bits in which its entries differ
+  if (!in_lds) {
+    const SegmentOut whole{p, n, values_out, indices_out, out_lo, lo_key};
+    const bool stored = store_equal_segment(seg_id, m, slot, parts, kk, ckey, cidx, cseg, whole, sh);
+    if (stored || slot != 0u) return;  // (keys that differ: the owner sorts, alone)
+  }
   __syncthreads();
 
   // One pass over the segment ids, then the segment's entries (key, inverted index) are fetched

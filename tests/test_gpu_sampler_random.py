@@ -111,6 +111,59 @@ def test_random_topk_sort_scatter(oracle, seed):
     assert np.array_equal(dw.cpu().numpy(), oracle.scatter_f32(w.copy(), uidx_np, uval))
 
 
+def _tied_values(rng, n, k):
+    """Priorities with masses of equal or nearly equal entries around and above the k-th largest:
+    one to five groups of 500 to 120 000 entries -- above everything, around the threshold, a
+    few ulps from another group, or anywhere in the selection -- scattered or as one stretch of
+    consecutive entries; or integers from a small range."""
+    if int(rng.integers(0, 4)) == 3:
+        return rng.integers(0, int(rng.integers(2, 3000)), size=n).astype(np.float32)
+    w = (rng.lognormal(0, 1, size=n) ** 0.6).astype(np.float32)
+    srt = np.sort(w)
+    thr = srt[n - k]
+    vals = []
+    for _ in range(int(rng.integers(1, 6))):
+        c = int(rng.integers(0, 4))
+        if c == 0:
+            v = np.float32(srt[-1] * rng.uniform(1.0, 3.0))
+        elif c == 1:
+            v = np.float32(thr * rng.uniform(0.98, 1.3))
+        elif c == 2 and vals:
+            v = (np.nextafter(vals[-1], np.float32(np.inf), dtype=np.float32) if rng.random() < 0.5
+                 else np.float32(vals[-1] * (1 + 1e-6 * rng.integers(1, 50))))
+        else:
+            v = np.float32(rng.uniform(thr, srt[-1]))
+        vals.append(np.float32(v))
+        size = int(rng.integers(500, min(120_000, n // 3)))
+        if rng.random() < 0.5:
+            w[rng.integers(0, n, size=size)] = v
+        else:
+            a = int(rng.integers(0, n - size))
+            w[a:a + size] = v
+    return w
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_random_topk_with_masses_of_ties(oracle, seed):
+    """Value order sorts by segments; a segment of thousands of equal priorities does not fit its
+    LDS buffers and takes the paths that keep index order instead of sorting by index."""
+    from gear_amd import ops
+    rng = np.random.default_rng(7000 + seed)
+    n = int(rng.integers(262_144, 4_000_000))
+    k = int(rng.integers(9_000, min(131_072, n // 8) + 1))
+    w = _tied_values(rng, n, k)
+    announce("random top-k with ties seed=%d n=%d k=%d" % (seed, n, k))
+    dw = _dev(w)
+    for by_value in (True, False):
+        vals, idx = ops.topk(dw, k, sorted_by_value=by_value)
+        torch.cuda.synchronize()
+        _, eidx = oracle.topk_f32(w, k, by_value)
+        assert np.array_equal(idx.cpu().numpy(), eidx)
+        assert np.array_equal(vals.cpu().numpy().view(np.uint32), w[eidx].view(np.uint32))
+    ref = np.argsort(-w.astype(np.float64), kind="stable")[:k]     # independent statement
+    assert np.array_equal(oracle.topk_f32(w, k, True)[1], ref)
+
+
 @pytest.mark.parametrize("seed", [3, 8, 13])
 def test_random_entry_points_with_workspaces_full_of_leftovers(oracle, seed, monkeypatch):
     """No entry point may depend on what its workspace held: every shared workspace is refilled
