@@ -1994,8 +1994,10 @@ __device__ __forceinline__ bool store_equal_segment(uint32_t seg_id, uint32_t m,
   const uint32_t w_end = w_begin + per_wave < kk ? w_begin + per_wave : kk;
   if (tid < 4) sh.bits_or_and[tid] = tid < 2 ? 0u : 0xffffffffu;
   __syncthreads();
+  // (bits_or_and[1] is raised by the first wave that sees two keys: the others stop looking)
+  volatile uint32_t *differ = &sh.bits_or_and[1];
   uint32_t cnt = 0, k_or = 0u, k_and = 0xffffffffu;
-  for (uint32_t c0 = w_begin; c0 < w_end; c0 += kWave * kLoadsAhead) {
+  for (uint32_t c0 = w_begin; c0 < w_end && *differ == 0u; c0 += kWave * kLoadsAhead) {
     uint8_t id[kLoadsAhead];
     uint32_t key[kLoadsAhead];
 #pragma unroll
@@ -2013,6 +2015,10 @@ __device__ __forceinline__ bool store_equal_segment(uint32_t seg_id, uint32_t m,
       k_or |= hit ? key[u] : 0u;
       k_and &= hit ? key[u] : 0xffffffffu;
     }
+    // (a lane's own keys, or two lanes' -- the wave's first hit against every other one)
+    const uint64_t has = wave_ballot(cnt != 0u);
+    const uint32_t first = (uint32_t)__builtin_amdgcn_readlane((int)k_or, has ? __builtin_ctzll(has) : 0);
+    if (wave_ballot(cnt != 0u && (k_or != k_and || k_or != first)) != 0ull && lane == 0) *differ = 1u;
   }
   cnt = (uint32_t)wave_sum((int)cnt);
   for (int d = 32; d >= 1; d >>= 1) {
@@ -2026,7 +2032,7 @@ __device__ __forceinline__ bool store_equal_segment(uint32_t seg_id, uint32_t m,
   }
   __syncthreads();
   const uint32_t key = sh.bits_or_and[0];
-  const bool equal = key == sh.bits_or_and[2];
+  const bool equal = key == sh.bits_or_and[2] && sh.bits_or_and[1] == 0u;
   uint32_t run = (uint32_t)wave_sum((int)(lane < wave ? sh.wsum[lane] : 0u));
   __syncthreads();  // (sh is used again by whoever goes on)
   if (!equal) return false;
